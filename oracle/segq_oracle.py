@@ -1,0 +1,556 @@
+"""CPU oracle for the real-quantized segmented linear.  TEST INFRASTRUCTURE ONLY.
+
+This file is a from-scratch numpy restatement of the arithmetic that the
+reference implements in CUDA/CUTLASS and in its torch "fake quant" path.  It
+is the checker for the HIP kernels: only tests, the smoke check and the bench's
+``cpu_baseline`` leg may import it.  Nothing in the shipped package does.
+
+Every public function names the reference file:line it restates.  Conventions
+taken from the reference:
+
+* a *scale* is multiplicative: ``code = round(x * scale)``, ``scale = qmax/amax``;
+  dequantisation divides by ``scale_x * scale_w``
+  (segquant/src/real_quant/quantizer.cuh:65, dequantizer.cuh:48).
+* activations are ``(S, ..., M, K)``, weights ``(S, N, K)`` (8-bit codes) or
+  ``(S, N*K/2)`` bytes (int4, low nibble = even element); a scale tensor with
+  ``numel == S`` is per segment, otherwise it is read flat as ``(S, M)`` /
+  ``(S, N)`` (segquant/src/real_quant/real_gemm.cu:644-670, :703, :743).
+
+How each function is pinned (none of it by importing the reference):
+
+=====================  =====================================================
+int8 / int4 codes      closed form + brute force over ties, limits, NaN, inf
+int4 pack / unpack     exhaustive over all nibble pairs, round trip
+e4m3 encode / decode   torch's ``float8_e4m3fn`` cast on clamped input, the
+                       exhaustive 256-entry decode table, every midpoint
+                       between neighbouring representable values
+int32 accumulators     brute-force triple loop on tiny shapes; fp64 BLAS is
+                       exact for these magnitudes
+dequant, bias          closed form
+segment semantics      concatenation / summation invariants
+scale formulas         closed forms incl. the 2^-24 epsilon and 127-vs-128
+fake-quant path        identities against the code path (dequantised codes)
+=====================  =====================================================
+
+The reference's own tests hold no golden vectors for this path, so the pins
+above are all there is.  Parity status of the pieces that exist only in this
+build and not in the reference (dynamic per-token scales, unequal K segments,
+group-wise int4 scales): closed form only.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+EPS = 1.0 / (1 << 24)  # segquant/quantizers/quantizer.py:167, :404
+
+FMT_INT8 = "int8"
+FMT_INT4 = "int4"
+FMT_E4M3 = "fpe4m3"
+
+
+# ---------------------------------------------------------------------------
+# float helpers
+# ---------------------------------------------------------------------------
+def _f32(x) -> np.ndarray:
+    return np.asarray(x, dtype=np.float32)
+
+
+def round_to_bf16(x) -> np.ndarray:
+    """fp32 -> nearest bf16 (ties to even), returned as fp32 values."""
+    x = np.ascontiguousarray(_f32(x))
+    u = x.view(np.uint32).astype(np.uint64)
+    nan = np.isnan(x)
+    lsb = (u >> 16) & 1
+    u = (u + 0x7FFF + lsb) & 0xFFFF0000
+    out = u.astype(np.uint32).view(np.float32).copy()
+    out[nan] = np.nan
+    return out.reshape(x.shape)
+
+
+def round_to_dtype(x, dtype: str) -> np.ndarray:
+    """Round fp32 values to the grid of ``dtype`` ("fp32" | "fp16" | "bf16")."""
+    if dtype == "fp32":
+        return _f32(x).copy()
+    if dtype == "fp16":
+        with np.errstate(over="ignore"):
+            return _f32(x).astype(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        return round_to_bf16(x)
+    raise ValueError(dtype)
+
+
+# ---------------------------------------------------------------------------
+# e4m3 (OCP "e4m3fn": bias 7, max 448, no inf, NaN = S.1111.111)
+# ---------------------------------------------------------------------------
+def e4m3_decode_table() -> np.ndarray:
+    """All 256 code values as fp32.  Codes 0x7F / 0xFF are NaN."""
+    t = np.zeros(256, dtype=np.float64)
+    for c in range(256):
+        s = -1.0 if c & 0x80 else 1.0
+        e = (c >> 3) & 0xF
+        m = c & 7
+        if e == 0xF and m == 7:
+            t[c] = np.nan
+        elif e == 0:
+            t[c] = s * m * 2.0 ** -9
+        else:
+            t[c] = s * (1.0 + m / 8.0) * 2.0 ** (e - 7)
+    return t.astype(np.float32)
+
+
+_E4M3_TABLE = e4m3_decode_table()
+
+
+def e4m3_decode(codes) -> np.ndarray:
+    return _E4M3_TABLE[np.asarray(codes, dtype=np.uint8)]
+
+
+def e4m3_encode(v) -> np.ndarray:
+    """fp32 -> e4m3 code: round to nearest even, saturate to +-448, NaN -> 0x7F.
+
+    Restates the hardware cast the reference relies on,
+    ``static_cast<__nv_fp8_e4m3>(float)`` (segquant/src/real_quant/quantizer.cuh:21-29,
+    segquant/src/fake_quant/quantizer_fp8.cpp:35-36).  The sign of a NaN is
+    dropped (0x7F), which is the value the reference's survey of that cast records.
+    """
+    v = _f32(v)
+    shape = v.shape
+    v = v.reshape(-1)
+    nan = np.isnan(v)
+    sign = np.signbit(v).astype(np.uint8) << 7
+    a = np.abs(v.astype(np.float64))
+    a = np.where(nan, 0.0, np.minimum(a, 448.0))
+    code = np.zeros(a.shape, dtype=np.int64)
+    sub = a < 2.0 ** -6
+    # subnormals: multiples of 2^-9; 8 * 2^-9 is the first normal and has code 8
+    code[sub] = np.rint(a[sub] * 2.0 ** 9).astype(np.int64)
+    nrm = ~sub
+    if nrm.any():
+        mant, ex = np.frexp(a[nrm])  # a = mant * 2^ex, mant in [0.5, 1)
+        e = ex.astype(np.int64) - 1
+        q = np.rint((mant * 2.0 - 1.0) * 8.0).astype(np.int64)
+        carry = q == 8
+        e = e + carry
+        q = np.where(carry, 0, q)
+        code[nrm] = ((e + 7) << 3) | q
+    out = code.astype(np.uint8) | sign
+    out[nan] = 0x7F
+    return out.reshape(shape)
+
+
+def e4m3_roundtrip(v) -> np.ndarray:
+    """``float(e4m3(v))`` -- the reference's fake_e4m3fy
+    (segquant/src/fake_quant/quantizer_fp8.cpp:25-39, quantizer_fp8.cu:34-41)."""
+    return e4m3_decode(e4m3_encode(v))
+
+
+# ---------------------------------------------------------------------------
+# integer codes (segquant/src/real_quant/quantizer.cuh:31-50)
+# ---------------------------------------------------------------------------
+def int8_codes(v) -> np.ndarray:
+    """``int8(rintf(fminf(fmaxf(v, -128), 127)))``; clamp first, then round half
+    to even.  fmaxf drops a NaN operand, so NaN becomes -128."""
+    v = _f32(v)
+    c = np.clip(np.where(np.isnan(v), np.float32(-128.0), v), -128.0, 127.0)
+    return np.rint(c).astype(np.int8)
+
+
+def int4_codes(v) -> np.ndarray:
+    """Signed 4-bit value in [-8, 7] (as int8), before packing."""
+    v = _f32(v)
+    c = np.clip(np.where(np.isnan(v), np.float32(-8.0), v), -8.0, 7.0)
+    return np.rint(c).astype(np.int8)
+
+
+def pack_int4(q) -> np.ndarray:
+    """Flat element i -> byte i/2; even i in the low nibble, odd i in the high
+    nibble, two's complement (segquant/src/real_quant/quantizer.cuh:37-50)."""
+    q = np.asarray(q, dtype=np.int8).reshape(-1)
+    if q.size % 2:
+        q = np.concatenate([q, np.zeros(1, np.int8)])
+    u = q.astype(np.uint8) & 0xF
+    return (u[0::2] | (u[1::2] << 4)).astype(np.uint8)
+
+
+def unpack_int4(b, n=None) -> np.ndarray:
+    """Inverse of :func:`pack_int4`; returns sign-extended int8 values."""
+    b = np.asarray(b, dtype=np.uint8).reshape(-1)
+    lo = (b & 0xF).astype(np.int8)
+    hi = (b >> 4).astype(np.int8)
+    lo = np.where(lo > 7, lo - 16, lo).astype(np.int8)
+    hi = np.where(hi > 7, hi - 16, hi).astype(np.int8)
+    out = np.empty(b.size * 2, dtype=np.int8)
+    out[0::2] = lo
+    out[1::2] = hi
+    return out if n is None else out[:n]
+
+
+def codes_of(v, fmt: str) -> np.ndarray:
+    """Scaled fp32 value -> storage code (int8, signed int4 value, or e4m3 byte)."""
+    if fmt == FMT_INT8:
+        return int8_codes(v)
+    if fmt == FMT_INT4:
+        return int4_codes(v)
+    if fmt == FMT_E4M3:
+        return e4m3_encode(v)
+    raise ValueError(fmt)
+
+
+def code_values(codes, fmt: str) -> np.ndarray:
+    """Numeric value of storage codes as fp64 (exact)."""
+    if fmt in (FMT_INT8, FMT_INT4):
+        return np.asarray(codes).astype(np.float64)
+    if fmt == FMT_E4M3:
+        return e4m3_decode(codes).astype(np.float64)
+    raise ValueError(fmt)
+
+
+# ---------------------------------------------------------------------------
+# scale indexing (quantizer.cuh:148-157, dequantizer.cuh:8-33)
+# ---------------------------------------------------------------------------
+def _expand_scale_x(scale_x, S: int, M: int) -> np.ndarray:
+    """-> (S, M, 1).  numel == S: one scale per segment, else flat (S, M)."""
+    s = _f32(scale_x).reshape(-1)
+    if s.size == S:
+        return np.broadcast_to(s.reshape(S, 1, 1), (S, M, 1))
+    if s.size != S * M:
+        raise ValueError(f"scale_x has {s.size} elements, expected {S} or {S * M}")
+    return s.reshape(S, M, 1)
+
+
+def _expand_scale_w(scale_w, S: int, N: int) -> np.ndarray:
+    """-> (S, 1, N).  numel == S: one scale per segment, else flat (S, N)."""
+    s = _f32(scale_w).reshape(-1)
+    if s.size == S:
+        return np.broadcast_to(s.reshape(S, 1, 1), (S, 1, N))
+    if s.size != S * N:
+        raise ValueError(f"scale_w has {s.size} elements, expected {S} or {S * N}")
+    return s.reshape(S, 1, N)
+
+
+# ---------------------------------------------------------------------------
+# activation / weight quantisation
+# ---------------------------------------------------------------------------
+def quantize_act(x, scale_x, fmt: str) -> np.ndarray:
+    """Activation codes, kernel K6 (segquant/src/real_quant/quantizer.cuh:159-176).
+
+    ``x`` is (S, ..., M, K) in any float dtype (converted to fp32 exactly);
+    returns codes of shape (S, M, K) (unpacked, also for int4).
+    """
+    x = np.asarray(x)
+    S, K = x.shape[0], x.shape[-1]
+    xf = x.astype(np.float32).reshape(S, -1, K)
+    M = xf.shape[1]
+    v = xf * _expand_scale_x(scale_x, S, M)  # fp32 * fp32 -> fp32
+    return codes_of(v, fmt)
+
+
+def quantize_act_dual(x, pos_scale_x, neg_scale_x, fmt: str):
+    """DualScale codes, kernel K7 (segquant/src/real_quant/quantizer.cuh:178-206).
+
+    ``x >= 0`` (which includes -0.0) takes the positive scale and leaves
+    code(0) in Xn; everything else (negatives and NaN) takes the negative scale
+    and leaves code(0) in Xp.  Returns (Xp, Xn), each (S, M, K).
+    """
+    x = np.asarray(x)
+    S, K = x.shape[0], x.shape[-1]
+    xf = x.astype(np.float32).reshape(S, -1, K)
+    M = xf.shape[1]
+    pos = xf >= 0
+    zero = codes_of(np.zeros((), np.float32), fmt)
+    cp = codes_of(xf * _expand_scale_x(pos_scale_x, S, M), fmt)
+    cn = codes_of(xf * _expand_scale_x(neg_scale_x, S, M), fmt)
+    xp = np.where(pos, cp, zero).astype(cp.dtype)
+    xn = np.where(pos, zero, cn).astype(cn.dtype)
+    return xp, xn
+
+
+def merge_dual_codes(xp, xn, x) -> np.ndarray:
+    """Single-tensor form of (Xp, Xn): the code of whichever branch was taken.
+
+    This layout exists only in this build (the reference stores both tensors);
+    it loses nothing because the untaken branch always holds code(0).
+    """
+    pos = np.asarray(x).astype(np.float32).reshape(xp.shape) >= 0
+    return np.where(pos, xp, xn).astype(xp.dtype)
+
+
+def quantize_weights(w, scale_w, fmt: str) -> np.ndarray:
+    """Weight codes, kernels K2/K4 (segquant/src/real_quant/quantizer.cuh:55-68,
+    :103-118; host side real_gemm.cu:538-638).  ``scale_w`` is a python float
+    (per tensor) or a vector with one entry per row of ``w`` (N, K).
+    Returns (N, K) codes (unpacked for int4)."""
+    w = np.asarray(w).astype(np.float32)
+    if np.ndim(scale_w) == 0:
+        v = w * np.float32(scale_w)
+    else:
+        s = _f32(scale_w).reshape(-1)
+        if s.size != w.shape[0]:
+            raise ValueError("per-row weight scale needs one entry per row")
+        v = w * s.reshape(-1, 1)
+    return codes_of(v, fmt)
+
+
+# ---------------------------------------------------------------------------
+# contraction (segquant/src/real_quant/real_gemm.cu:208-305)
+# ---------------------------------------------------------------------------
+def gemm_acc(a_codes, b_codes, fmt_a: str, fmt_b: str) -> np.ndarray:
+    """``acc[m, n] = sum_k A[m, k] * B[n, k]`` as fp64.
+
+    Exact for integer codes: |acc| <= K * 128 * 128 < 2^53, and fp64 BLAS adds
+    integers below 2^53 without rounding, so the result equals the int32
+    accumulator bit for bit.  For e4m3 every product is exact in fp32 and the
+    fp64 sum is the reference value that fp32 accumulation is compared against.
+    """
+    a = code_values(a_codes, fmt_a)
+    b = code_values(b_codes, fmt_b)
+    return a @ b.T
+
+
+def gemm_acc_bruteforce(a_codes, b_codes) -> np.ndarray:
+    """Triple loop in python ints; pins :func:`gemm_acc` on tiny shapes."""
+    a = np.asarray(a_codes).astype(np.int64)
+    b = np.asarray(b_codes).astype(np.int64)
+    M, K = a.shape
+    N = b.shape[0]
+    out = np.zeros((M, N), dtype=np.int64)
+    for m in range(M):
+        for n in range(N):
+            s = 0
+            for k in range(K):
+                s += int(a[m, k]) * int(b[n, k])
+            out[m, n] = s
+    return out
+
+
+# ---------------------------------------------------------------------------
+# dequantisation (segquant/src/real_quant/dequantizer.cuh:35-74)
+# ---------------------------------------------------------------------------
+def dequant(acc, scale_x, scale_w, out_dtype: str = "fp32") -> np.ndarray:
+    """``T(float(acc) / (sx * sw))`` for acc of shape (S, M, N), kernel K8."""
+    acc = np.asarray(acc)
+    S, M, N = acc.shape
+    yq = acc.astype(np.float32)
+    s = _expand_scale_x(scale_x, S, M) * _expand_scale_w(scale_w, S, N)  # fp32 product
+    return round_to_dtype(yq / s, out_dtype)
+
+
+def dequant_dual(acc_p, acc_n, pos_scale_x, neg_scale_x, scale_w, out_dtype: str = "fp32") -> np.ndarray:
+    """``T(Yp/(pos*sw) + Yn/(neg*sw))``, fp32 sum, one rounding; kernel K9."""
+    acc_p = np.asarray(acc_p)
+    S, M, N = acc_p.shape
+    sw = _expand_scale_w(scale_w, S, N)
+    yp = acc_p.astype(np.float32) / (_expand_scale_x(pos_scale_x, S, M) * sw)
+    yn = np.asarray(acc_n).astype(np.float32) / (_expand_scale_x(neg_scale_x, S, M) * sw)
+    return round_to_dtype(yp + yn, out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# host pipelines H1 / H2 (segquant/src/real_quant/real_gemm.cu:643-894)
+# ---------------------------------------------------------------------------
+def _weight_values(weights, S: int, K: int, fmt_w: str) -> np.ndarray:
+    w = np.asarray(weights)
+    if fmt_w == FMT_INT4:
+        wb = w.reshape(S, -1)
+        N = wb.shape[1] * 2 // K  # real_gemm.cu:670
+        return np.stack([unpack_int4(wb[s]).reshape(N, K) for s in range(S)])
+    return w.reshape(S, -1, K)
+
+
+def real_quantized_gemm_scaled(inputs, weights, scale_x, scale_w, fmt_a: str, fmt_w: str,
+                               out_dtype: str = "fp32", return_acc: bool = False):
+    """The reference's ``<prefix>_real_quantized_gemm_scaled`` end to end
+    (segquant/src/real_quant/real_gemm.cu:643-750): quantise the activations,
+    contract each segment with its weight codes, dequantise.  ``inputs`` is
+    (S, ..., M, K); the result is (S, ..., M, N) holding values on the grid of
+    ``out_dtype``.  The scalar fast path (:707-712) multiplies by a reciprocal
+    instead of dividing; that differs from this formula by at most one fp32 ulp
+    and is not modelled separately."""
+    x = np.asarray(inputs)
+    S, K = x.shape[0], x.shape[-1]
+    xq = quantize_act(x, scale_x, fmt_a)
+    wv = _weight_values(weights, S, K, fmt_w)
+    acc = np.stack([gemm_acc(xq[s], wv[s], fmt_a, fmt_w) for s in range(S)])
+    out = dequant(acc, scale_x, scale_w, out_dtype).reshape(*x.shape[:-1], wv.shape[1])
+    return (out, acc) if return_acc else out
+
+
+def real_quantized_gemm_dual_scaled(inputs, weights, pos_scale_x, neg_scale_x, scale_w,
+                                    fmt_a: str, fmt_w: str, out_dtype: str = "fp32",
+                                    return_acc: bool = False):
+    """The reference's ``<prefix>_real_quantized_gemm_dual_scaled``
+    (segquant/src/real_quant/real_gemm.cu:752-894)."""
+    x = np.asarray(inputs)
+    S, K = x.shape[0], x.shape[-1]
+    xp, xn = quantize_act_dual(x, pos_scale_x, neg_scale_x, fmt_a)
+    wv = _weight_values(weights, S, K, fmt_w)
+    acc_p = np.stack([gemm_acc(xp[s], wv[s], fmt_a, fmt_w) for s in range(S)])
+    acc_n = np.stack([gemm_acc(xn[s], wv[s], fmt_a, fmt_w) for s in range(S)])
+    out = dequant_dual(acc_p, acc_n, pos_scale_x, neg_scale_x, scale_w, out_dtype)
+    out = out.reshape(*x.shape[:-1], wv.shape[1])
+    return (out, acc_p, acc_n) if return_acc else out
+
+
+def recombine(out_chunks, seg_mode: str, bias=None, out_dtype: str = "fp32") -> np.ndarray:
+    """Tail of ``SegmentLinear.forward`` (segquant/layers/SegmentLinear.py:228-241).
+
+    weight-seg: (S, ..., n) -> (..., S*n).  input-seg: sum over S, done in the
+    output dtype as the reference does.  Bias is added in the output dtype.
+    """
+    o = np.asarray(out_chunks, dtype=np.float32)
+    if seg_mode == "weight":
+        res = np.moveaxis(o, 0, -2).reshape(*o.shape[1:-1], -1)
+    elif seg_mode == "input":
+        res = o[0]
+        for s in range(1, o.shape[0]):
+            res = round_to_dtype(res + o[s], out_dtype)
+    else:
+        raise ValueError(seg_mode)
+    if bias is not None:
+        res = round_to_dtype(res + _f32(bias), out_dtype)
+    return res
+
+
+# ---------------------------------------------------------------------------
+# scale formulas (segquant/quantizers/quantizer.py:161-248, :398-452)
+# ---------------------------------------------------------------------------
+def int_qrange(bits: int):
+    return -(2 ** (bits - 1)), 2 ** (bits - 1) - 1  # quantizer.py:151-152
+
+
+def int_scale(amax, bits: int = 8):
+    """Symmetric per-tensor: ``qmax/amax`` if amax > eps else 1.0 (python float
+    arithmetic, quantizer.py:206-210).  Array input: ``qmax / clamp(amax, eps)``
+    in fp32 (quantizer.py:211-219)."""
+    _, qmax = int_qrange(bits)
+    if np.ndim(amax) == 0:
+        amax = float(amax)
+        return qmax / amax if amax > EPS else 1.0
+    return (np.float32(qmax) / np.maximum(_f32(amax), np.float32(EPS))).astype(np.float32)
+
+
+def int_dual_scales(pos_amax, neg_amax, bits: int = 8):
+    """``pos = qmax/pos_amax``, ``neg = qmin/(-neg_amax)`` (quantizer.py:170-203)."""
+    qmin, qmax = int_qrange(bits)
+    if np.ndim(pos_amax) == 0:
+        pos_amax, neg_amax = float(pos_amax), float(neg_amax)
+        neg = qmin / (-neg_amax) if neg_amax > EPS else 1.0
+        pos = qmax / pos_amax if pos_amax > EPS else 1.0
+        return pos, neg
+    neg = np.float32(qmin) / (-np.maximum(_f32(neg_amax), np.float32(EPS)))
+    pos = np.float32(qmax) / np.maximum(_f32(pos_amax), np.float32(EPS))
+    return pos.astype(np.float32), neg.astype(np.float32)
+
+
+def fp8_scale(amax):
+    """``448/amax`` with the same epsilon rules (quantizer.py:437-452)."""
+    if np.ndim(amax) == 0:
+        amax = float(amax)
+        return 448.0 / amax if amax > EPS else 1.0
+    return (np.float32(448.0) / np.maximum(_f32(amax), np.float32(EPS))).astype(np.float32)
+
+
+def fp8_dual_scales(pos_amax, neg_amax):
+    """448 on both sides (quantizer.py:406-436)."""
+    return fp8_scale(pos_amax), fp8_scale(neg_amax)
+
+
+def dual_amax(x, axis=None):
+    """Strict masks ``x > 0`` / ``x < 0``; an empty side has amax 0
+    (quantizer.py:172-189)."""
+    x = _f32(x)
+    pos = np.where(x > 0, np.abs(x), 0.0)
+    neg = np.where(x < 0, np.abs(x), 0.0)
+    if axis is None:
+        return float(pos.max()), float(neg.max())
+    return pos.max(axis=axis), neg.max(axis=axis)
+
+
+# ---------------------------------------------------------------------------
+# fake-quant reference path (segquant/quantizers/quantizer.py:250-281, :462-528)
+# ---------------------------------------------------------------------------
+def fake_quant_int(x, scale, bits: int = 8) -> np.ndarray:
+    """``clamp(round(x*s), qmin, qmax) / s`` in fp32 (quantizer.py:277-281;
+    symmetric, zero point 0)."""
+    qmin, qmax = int_qrange(bits)
+    x = _f32(x)
+    s = _f32(scale)
+    return (np.clip(np.rint(x * s), qmin, qmax) / s).astype(np.float32)
+
+
+def fake_quant_int_dual(x, pos_scale, neg_scale, bits: int = 8) -> np.ndarray:
+    """quantizer.py:259-265."""
+    qmin, qmax = int_qrange(bits)
+    x = _f32(x)
+    ps, ns = _f32(pos_scale), _f32(neg_scale)
+    q = np.where(x >= 0, np.clip(np.rint(x * ps), 0, qmax), np.clip(np.rint(x * ns), qmin, 0))
+    return np.where(x >= 0, q / ps, q / ns).astype(np.float32)
+
+
+def simulate_fp(x, fp_min: float, fp_max: float, mant_bits: int) -> np.ndarray:
+    """The reference's pure-torch float simulation, which has no subnormals:
+    anything below ``fp_min`` becomes zero (quantizer.py:462-482)."""
+    x = _f32(x)
+    a = np.minimum(np.abs(x), np.float32(fp_max))
+    a = np.where(a < fp_min, np.float32(0), a)
+    expo = np.floor(np.log2(np.maximum(a, np.float32(fp_min))))
+    mant = a / np.exp2(expo)
+    mant_r = np.rint((mant - 1) * 2 ** mant_bits) / 2 ** mant_bits
+    return ((1 + mant_r) * np.exp2(expo) * np.sign(x)).astype(np.float32)
+
+
+E4M3_FP_MIN = (2.0 ** -6) * (240 / 448.0)  # quantizer.py:384
+
+
+def fake_quant_fp8(x, scale, simulate: str = "e4m3") -> np.ndarray:
+    """``e4m3(x*s)/s`` with ``|x| < 2^-24 -> 0`` (quantizer.py:484-528).
+    ``simulate="e4m3"`` is the branch taken when the fake_e4m3fy extension is
+    present; ``"simulate_fp"`` is the pure-torch fallback."""
+    x = _f32(x)
+    s = _f32(scale)
+    v = x * s
+    if simulate == "e4m3":
+        q = e4m3_roundtrip(v)
+    else:
+        q = simulate_fp(v, E4M3_FP_MIN, 448.0, 3)
+    out = (q / s).astype(np.float32)
+    return np.where(np.abs(x) < EPS, np.float32(0), out)
+
+
+def fake_quant_fp8_dual(x, pos_scale, neg_scale) -> np.ndarray:
+    """quantizer.py:487-507 (e4m3 branch)."""
+    x = _f32(x)
+    ps, ns = _f32(pos_scale), _f32(neg_scale)
+    v = np.where(x >= 0, x * ps, x * ns)
+    q = e4m3_roundtrip(v)
+    out = np.where(x >= 0, q / ps, q / ns).astype(np.float32)
+    return np.where(np.abs(x) < EPS, np.float32(0), out)
+
+
+def segmented_matmul(a, b) -> np.ndarray:
+    """``a @ b^T`` per segment with leading-dim broadcast
+    (segquant/layers/segment_tensor_manager.py:83-94).  a (S, ..., K), b (S, N, K)."""
+    a = _f32(a)
+    b = _f32(b)
+    bt = np.swapaxes(b, -1, -2)
+    while bt.ndim < a.ndim:
+        bt = np.expand_dims(bt, 1)
+    return a @ bt
+
+
+def segment_views(x, w, seg_mode: str, chunks: int):
+    """Segment views of the input and the weight
+    (segquant/layers/segment_tensor_manager.py:15-23, :45-51).
+    Returns (x_seg (S, ..., k), w_seg (S, n, k))."""
+    x = np.asarray(x)
+    w = np.asarray(w)
+    N, K = w.shape
+    if seg_mode == "weight":
+        xs = np.broadcast_to(x[None], (chunks, *x.shape))
+        ws = w.reshape(chunks, N // chunks, K)
+    elif seg_mode == "input":
+        xs = np.moveaxis(x.reshape(*x.shape[:-1], chunks, K // chunks), -2, 0)
+        ws = np.moveaxis(w.reshape(N, chunks, K // chunks), 1, 0)
+    else:
+        raise ValueError(seg_mode)
+    return xs, ws

@@ -1,0 +1,287 @@
+"""Pins for the CPU oracle: closed forms, library routines, brute force.
+
+None of these tests retypes the oracle's own formula; each compares it with an
+independent source (torch's float8 cast, python integer arithmetic, an
+exhaustive table, an algebraic invariant).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import segq_oracle as O
+
+
+# ------------------------------------------------------------------ e4m3
+def test_e4m3_table_matches_torch_decode():
+    codes = torch.arange(256, dtype=torch.uint8)
+    ref = codes.view(torch.float8_e4m3fn).float().numpy()
+    tab = O.e4m3_decode_table()
+    assert np.array_equal(np.isnan(ref), np.isnan(tab))
+    ok = ~np.isnan(ref)
+    assert np.array_equal(ref[ok], tab[ok])
+    assert tab[0x7E] == 448.0 and tab[0x08] == 2.0 ** -6 and tab[0x01] == 2.0 ** -9
+
+
+def test_e4m3_encode_is_identity_on_representable_values():
+    tab = O.e4m3_decode_table()
+    codes = np.arange(256, dtype=np.uint8)
+    ok = ~np.isnan(tab)
+    enc = O.e4m3_encode(tab[ok])
+    # -0.0 keeps its sign bit (0x80)
+    assert np.array_equal(enc, codes[ok])
+
+
+def test_e4m3_midpoints_round_to_even_mantissa():
+    tab = O.e4m3_decode_table()
+    pos = np.sort(tab[:0x7F])  # 0 .. 448, ascending, codes 0..0x7E
+    for c in range(0x7E):
+        lo, hi = float(pos[c]), float(pos[c + 1])
+        mid = np.float32((lo + hi) / 2)  # exact in fp32
+        want = c if c % 2 == 0 else c + 1
+        assert O.e4m3_encode(mid) == want, (c, mid)
+        assert O.e4m3_encode(-mid) == (want | 0x80)
+        below = np.nextafter(mid, np.float32(0))
+        above = np.nextafter(mid, np.float32(1e9))
+        assert O.e4m3_encode(below) == c
+        assert O.e4m3_encode(above) == c + 1
+
+
+def test_e4m3_encode_matches_torch_cast_on_clamped_input():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(200000, generator=g) * torch.exp(torch.randn(200000, generator=g) * 4)
+    x = torch.cat([x, torch.tensor([0.0, -0.0, 448.0, 449.0, 464.0, 465.0, 1e9, -1e9,
+                                    2.0 ** -10, 2.0 ** -9, 3 * 2.0 ** -10, 2.0 ** -6, 17., 19., 21., 23.])])
+    ref = torch.clamp(x, -448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = O.e4m3_encode(x.numpy())
+    assert np.array_equal(ref, got)
+
+
+def test_e4m3_special_values():
+    assert O.e4m3_encode(np.float32("nan")) == 0x7F
+    assert O.e4m3_encode(np.float32("inf")) == 0x7E
+    assert O.e4m3_encode(np.float32("-inf")) == 0xFE
+    assert O.e4m3_encode(np.float32(1e30)) == 0x7E
+    assert O.e4m3_encode(np.float32(2.0 ** -10)) == 0  # tie to even (0)
+    assert O.e4m3_encode(np.float32(3 * 2.0 ** -10)) == 2  # tie between 1 and 2 -> 2
+
+
+def test_simulate_fp_agrees_with_e4m3_for_normals_only():
+    g = np.random.default_rng(3)
+    x = (g.standard_normal(50000) * 50).astype(np.float32)
+    x = x[np.abs(x) >= 2.0 ** -6]
+    a = O.simulate_fp(x, O.E4M3_FP_MIN, 448.0, 3)
+    b = O.e4m3_roundtrip(x)
+    # rint in simulate_fp is also half-to-even, so they agree on normals
+    assert np.array_equal(a, b)
+    # subnormal range: e4m3 keeps multiples of 2^-9, simulate_fp flushes below fp_min
+    tiny = np.float32(2.0 ** -8)
+    assert O.e4m3_roundtrip(tiny) == tiny
+    assert O.simulate_fp(tiny, O.E4M3_FP_MIN, 448.0, 3) == 0
+
+
+# ------------------------------------------------------------------ int codes
+def test_int8_codes_ties_limits_specials():
+    v = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, 127.49, -127.5, -128.5, 1e9, -1e9,
+                  np.inf, -np.inf, np.nan, 0.0, -0.0], dtype=np.float32)
+    want = [0, 2, 2, 0, -2, -2, 126, 127, 127, -128, -128, 127, -128, 127, -128, -128, 0, 0]
+    assert O.int8_codes(v).tolist() == want
+
+
+def test_int8_codes_equal_python_round_on_dense_sweep():
+    v = np.linspace(-140, 140, 56001, dtype=np.float32)
+    want = [int(max(-128, min(127, round(float(t))))) for t in v]  # python round is half-even
+    assert O.int8_codes(v).tolist() == want
+
+
+def test_int8_clamp_then_round_equals_round_then_clamp():
+    # the fake path rounds first and clamps after (quantizer.py:277-278); the
+    # kernel clamps first.  Integer bounds make them equal.
+    g = np.random.default_rng(0)
+    v = (g.standard_normal(100000) * 100).astype(np.float32)
+    assert np.array_equal(O.int8_codes(v), np.clip(np.rint(v), -128, 127).astype(np.int8))
+
+
+def test_int4_codes_and_pack_exhaustive():
+    v = np.array([-9, -8.5, -8, -7.5, -0.5, 0.5, 6.5, 7, 7.5, 8, np.nan], dtype=np.float32)
+    assert O.int4_codes(v).tolist() == [-8, -8, -8, -8, 0, 0, 6, 7, 7, 7, -8]
+    for lo in range(-8, 8):
+        for hi in range(-8, 8):
+            b = O.pack_int4(np.array([lo, hi], dtype=np.int8))
+            assert b.shape == (1,)
+            assert int(b[0]) == ((lo & 0xF) | ((hi & 0xF) << 4))
+            assert O.unpack_int4(b).tolist() == [lo, hi]
+    q = np.random.default_rng(1).integers(-8, 8, size=4096).astype(np.int8)
+    assert np.array_equal(O.unpack_int4(O.pack_int4(q)), q)
+
+
+# ------------------------------------------------------------------ contraction
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_INT4])
+def test_gemm_acc_matches_bruteforce(fmt):
+    g = np.random.default_rng(5)
+    lo, hi = (-128, 128) if fmt == O.FMT_INT8 else (-8, 8)
+    a = g.integers(-128, 128, size=(5, 48)).astype(np.int8)
+    b = g.integers(lo, hi, size=(7, 48)).astype(np.int8)
+    a[0, :] = -128
+    b[0, :] = lo
+    acc = O.gemm_acc(a, b, O.FMT_INT8, fmt)
+    assert np.array_equal(acc.astype(np.int64), O.gemm_acc_bruteforce(a, b))
+
+
+def test_gemm_acc_extreme_magnitude_is_exact():
+    K = 15360
+    a = np.full((2, K), -128, dtype=np.int8)
+    b = np.full((3, K), -128, dtype=np.int8)
+    acc = O.gemm_acc(a, b, O.FMT_INT8, O.FMT_INT8)
+    assert (acc == K * 128 * 128).all() and K * 128 * 128 < 2 ** 31
+
+
+def test_gemm_acc_equals_torch_int32_matmul():
+    g = torch.Generator().manual_seed(11)
+    a = torch.randint(-128, 128, (33, 256), generator=g, dtype=torch.int32)
+    b = torch.randint(-128, 128, (17, 256), generator=g, dtype=torch.int32)
+    ref = (a @ b.T).numpy()
+    acc = O.gemm_acc(a.numpy().astype(np.int8), b.numpy().astype(np.int8), O.FMT_INT8, O.FMT_INT8)
+    assert np.array_equal(acc.astype(np.int32), ref)
+
+
+def test_fp8_products_are_exact_in_fp32():
+    t = O.e4m3_decode_table()
+    t = t[~np.isnan(t)].astype(np.float64)
+    p = np.outer(t, t)
+    assert np.array_equal(p.astype(np.float32).astype(np.float64), p)
+
+
+# ------------------------------------------------------------------ scale indexing
+def test_scale_broadcast_rule_and_flat_indices():
+    S, B, M, K, N = 3, 2, 4, 16, 5
+    g = np.random.default_rng(2)
+    x = g.standard_normal((S, B, M, K)).astype(np.float32)
+    per_seg = np.array([1.0, 2.0, 4.0], dtype=np.float32)
+    per_tok = (np.arange(S * B * M) + 1).astype(np.float32)
+    c1 = O.quantize_act(x, per_seg, O.FMT_INT8)
+    c2 = O.quantize_act(x, per_tok, O.FMT_INT8)
+    xf = x.reshape(S, B * M, K)
+    for s in range(S):
+        for t in range(B * M):
+            assert np.array_equal(c1[s, t], O.int8_codes(xf[s, t] * per_seg[s]))
+            assert np.array_equal(c2[s, t], O.int8_codes(xf[s, t] * per_tok[s * B * M + t]))
+    acc = g.integers(-1000, 1000, size=(S, B * M, N))
+    sw = (np.arange(S * N) + 1).astype(np.float32)
+    y = O.dequant(acc, per_tok, sw)
+    for s in range(S):
+        for t in range(B * M):
+            for n in range(N):
+                want = np.float32(acc[s, t, n]) / (per_tok[s * B * M + t] * sw[s * N + n])
+                assert y[s, t, n] == np.float32(want)
+
+
+# ------------------------------------------------------------------ dual scale
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3, O.FMT_INT4])
+def test_dual_split_invariants(fmt):
+    g = np.random.default_rng(9)
+    x = g.standard_normal((1, 6, 32)).astype(np.float32)
+    x[0, 0, :4] = [0.0, -0.0, 1e-30, -1e-30]
+    xp, xn = O.quantize_act_dual(x, np.float32([30.0]), np.float32([50.0]), fmt)
+    vp, vn = O.code_values(xp, fmt), O.code_values(xn, fmt)
+    assert (vp * vn == 0).all() and (vp >= 0).all() and (vn <= 0).all()
+    # x == 0 (either sign) goes to the positive branch: Xn holds code(0)
+    assert (vn[0, 0, :2] == 0).all()
+    merged = O.merge_dual_codes(xp, xn, x)
+    assert np.array_equal(O.code_values(merged, fmt), vp + vn)
+
+
+def test_dual_with_equal_scales_reduces_to_single_scale_accumulator():
+    g = np.random.default_rng(4)
+    x = g.standard_normal((1, 9, 64)).astype(np.float32)
+    w = g.integers(-128, 128, size=(1, 11, 64)).astype(np.int8)
+    s = np.float32([40.0])
+    _, acc = O.real_quantized_gemm_scaled(x, w, s, np.float32([1.0]), O.FMT_INT8, O.FMT_INT8, return_acc=True)
+    _, ap, an = O.real_quantized_gemm_dual_scaled(x, w, s, s, np.float32([1.0]), O.FMT_INT8, O.FMT_INT8,
+                                                  return_acc=True)
+    assert np.array_equal(ap + an, acc)
+
+
+# ------------------------------------------------------------------ segments
+def test_weight_seg_is_concat_and_input_seg_is_sum():
+    g = np.random.default_rng(6)
+    M, K, N, S = 7, 64, 12, 2
+    x = g.standard_normal((M, K)).astype(np.float32)
+    wq = g.integers(-128, 128, size=(N, K)).astype(np.int8)
+    sx = np.float32([25.0])
+    # unsegmented accumulators
+    _, acc = O.real_quantized_gemm_scaled(x[None], wq[None], sx, np.float32([1.0]), O.FMT_INT8, O.FMT_INT8,
+                                          return_acc=True)
+    xs, ws = O.segment_views(x, wq, "weight", S)
+    _, acc_w = O.real_quantized_gemm_scaled(xs, ws, np.repeat(sx, S), np.ones(S, np.float32), O.FMT_INT8,
+                                            O.FMT_INT8, return_acc=True)
+    assert np.array_equal(np.concatenate(list(acc_w), axis=-1), acc[0])
+    xs, ws = O.segment_views(x, wq, "input", S)
+    _, acc_i = O.real_quantized_gemm_scaled(xs, ws, np.repeat(sx, S), np.ones(S, np.float32), O.FMT_INT8,
+                                            O.FMT_INT8, return_acc=True)
+    assert np.array_equal(acc_i.sum(0), acc[0])
+    out = np.arange(S * M * 3, dtype=np.float32).reshape(S, M, 3)
+    assert np.array_equal(O.recombine(out, "weight"), np.concatenate([out[0], out[1]], axis=-1))
+    assert np.array_equal(O.recombine(out, "input", bias=np.ones(3, np.float32)), out[0] + out[1] + 1)
+
+
+# ------------------------------------------------------------------ scales
+def test_scale_closed_forms():
+    assert O.int_scale(2.0) == 63.5 and O.int_scale(0.0) == 1.0 and O.int_scale(2.0 ** -25) == 1.0
+    assert O.int_scale(3.5, bits=4) == 2.0
+    pos, neg = O.int_dual_scales(2.0, 4.0)
+    assert pos == 63.5 and neg == 32.0  # 127 on the positive side, 128 on the negative
+    pos, neg = O.int_dual_scales(0.0, 0.0)
+    assert pos == 1.0 and neg == 1.0
+    assert O.fp8_scale(7.0) == 64.0 and O.fp8_dual_scales(7.0, 14.0) == (64.0, 32.0)
+    v = O.int_scale(np.float32([0.0, 1.0]))
+    assert v[0] == np.float32(127.0) / np.float32(2.0 ** -24) and v[1] == 127.0
+    p, n = O.dual_amax(np.float32([[-3, 0, 2], [0, 0, 0]]), axis=-1)
+    assert p.tolist() == [2, 0] and n.tolist() == [3, 0]
+    assert O.dual_amax(np.float32([1, 2])) == (2.0, 0.0)
+
+
+# ------------------------------------------------------------------ fake quant vs code path
+def test_fake_int_equals_dequantised_codes():
+    g = np.random.default_rng(8)
+    x = (g.standard_normal((64, 96)) * 3).astype(np.float32)
+    s = np.float32(O.int_scale(float(np.abs(x).max())))
+    codes = O.int8_codes(x * s)
+    assert np.array_equal(O.fake_quant_int(x, s), codes.astype(np.float32) / s)
+    pa, na = O.dual_amax(x)
+    ps, ns = (np.float32(t) for t in O.int_dual_scales(pa, na))
+    xp, xn = O.quantize_act_dual(x[None], [ps], [ns], O.FMT_INT8)
+    want = np.where(x >= 0, xp[0].astype(np.float32) / ps, xn[0].astype(np.float32) / ns)
+    assert np.array_equal(O.fake_quant_int_dual(x, ps, ns), want)
+
+
+def test_fake_fp8_equals_dequantised_codes_and_zero_mask():
+    g = np.random.default_rng(10)
+    x = g.standard_normal((32, 64)).astype(np.float32)
+    x[0, 0] = 2.0 ** -26
+    s = np.float32(O.fp8_scale(float(np.abs(x).max())))
+    fq = O.fake_quant_fp8(x, s)
+    assert fq[0, 0] == 0
+    want = O.e4m3_decode(O.e4m3_encode(x * s)) / s
+    want[0, 0] = 0
+    assert np.array_equal(fq, want)
+
+
+def test_real_pipeline_matches_fake_path_within_tolerance():
+    g = np.random.default_rng(12)
+    M, K, N = 16, 128, 24
+    x = g.standard_normal((M, K)).astype(np.float32)
+    w = (g.standard_normal((N, K)) * 0.02).astype(np.float32)
+    sx = np.float32(O.int_scale(float(np.abs(x).max())))
+    sw = np.float32(O.int_scale(float(np.abs(w).max())))
+    wq = O.quantize_weights(w, float(sw), O.FMT_INT8)
+    y = O.real_quantized_gemm_scaled(x[None], wq[None], [sx], [sw], O.FMT_INT8, O.FMT_INT8)[0]
+    ref = O.segmented_matmul(O.fake_quant_int(x, sx)[None], O.fake_quant_int(w, sw)[None])[0]
+    assert np.abs(y - ref).max() <= 1e-3 * np.abs(ref).max()
+
+
+def test_round_to_bf16_matches_torch():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(100000, generator=g) * 100
+    assert np.array_equal(O.round_to_bf16(x.numpy()), x.to(torch.bfloat16).float().numpy())
