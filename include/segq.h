@@ -1,0 +1,205 @@
+/*
+ * libsegq -- C ABI of the MI355X (gfx950) real-quantized segmented linear.
+ *
+ * Plain pointers and sizes only; no torch types.  Every pointer named "device"
+ * is HIP device memory on the current device.  No entry point allocates,
+ * frees, synchronises or throws: each enqueues its kernels on the stream it is
+ * given and returns 0, or returns a non-zero segq_status and leaves a message
+ * for segq_last_error().
+ *
+ * Scale convention (the reference's): a scale is multiplicative,
+ * code = round(x * scale); de-quantisation divides by scale_x * scale_w
+ * (segquant/src/real_quant/quantizer.cuh:65, dequantizer.cuh:48).
+ */
+#ifndef SEGQ_H
+#define SEGQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* segq_stream_t; /* a hipStream_t; NULL is the default stream */
+
+enum segq_status {
+    SEGQ_OK = 0,
+    SEGQ_ERR_ARG = 1,         /* bad pointer, size, alignment or enum */
+    SEGQ_ERR_UNSUPPORTED = 2, /* a combination this build has no kernel for */
+    SEGQ_ERR_LAUNCH = 3       /* the HIP runtime refused the launch */
+};
+
+/* float element types of inputs, outputs and bias.  Mirrors the dtypes the
+ * reference dispatches over (segquant/src/real_quant/real_gemm.cu:22-28). */
+enum segq_dtype {
+    SEGQ_F32 = 0,
+    SEGQ_F16 = 1,
+    SEGQ_BF16 = 2,
+    SEGQ_ACC = 3 /* GEMM output only: the raw accumulator, int32 (integer codes) or fp32 (e4m3) */
+};
+
+/* storage formats of codes.  Mirrors StoreType<> (segquant/src/real_quant/seg_utils.h:25-45):
+ * int8 travels as int8, e4m3 as one byte, int4 as two values per byte with the
+ * even element in the low nibble (segquant/src/real_quant/quantizer.cuh:37-50). */
+enum segq_code {
+    SEGQ_CODE_I8 = 0,
+    SEGQ_CODE_E4M3 = 1,
+    SEGQ_CODE_I4 = 2
+};
+
+#define SEGQ_MAX_KSEG 8
+#define SEGQ_MAX_RANGES 16
+
+int segq_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* segq_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Quantise a row-major float matrix to codes.
+ *
+ * Replaces the reference's quantise kernels and their launches:
+ *   activations  real_quantize_scaled_kernel / real_quantize_dual_scaled_kernel,
+ *                segment form (segquant/src/real_quant/quantizer.cuh:148-206),
+ *                launched from real_gemm.cu:701-705 and :818-826;
+ *   weights      the scalar and per-row forms (quantizer.cuh:55-68, :103-118)
+ *                behind real_quantized_quantize_weights (real_gemm.cu:538-638).
+ *
+ * The scale of element (row, col) is
+ *     scale[(row / seg_rows) * seg_stride + (row % seg_rows) * row_stride
+ *           + kseg(col) * kseg_stride]
+ * where kseg(col) is the index of the column segment that holds col.  With the
+ * reference's (S, ..., M, K) activations flattened to rows = S*M, seg_rows = M:
+ * a per-segment scale tensor is {seg_stride 1, row_stride 0}, a per-token one
+ * is {seg_stride M, row_stride 1} (quantizer.cuh:148-157).
+ *
+ * dual != 0 selects DualScale (quantizer.cuh:178-206): x >= 0 uses scale[],
+ * anything else uses scale_neg[] at the same index.  Bit i of dual_kseg_mask
+ * says whether column segment i is dual; other segments use scale[] for both
+ * signs.  With codes_neg == NULL one merged code tensor is written (the code of
+ * the branch that was taken); with codes_neg != NULL the reference's two
+ * tensors are written, Xp to codes and Xn to codes_neg.
+ *
+ * dynamic != 0: scale[] (and scale_neg[]) are OUTPUTS.  The kernel takes the
+ * absolute maximum of every (row, column segment), writes
+ * qmax / max(amax, 2^-24) there (segquant/quantizers/quantizer.py:211-219;
+ * dual: :183-203; e4m3: 448) and quantises with it.  Needs row_stride == 1 or a
+ * single row per scale; has no counterpart kernel in the reference, whose
+ * dynamic mode calls a method that does not exist (optimum/optimizer.py:96-100).
+ * ---------------------------------------------------------------------- */
+typedef struct segq_quant_desc {
+    const void* x;      /* device, rows x cols, x_dtype, row stride ldx elements */
+    int32_t x_dtype;    /* segq_dtype: F32 | F16 | BF16 */
+    int32_t code_fmt;   /* segq_code */
+    int64_t rows;
+    int64_t cols;       /* multiple of 16 */
+    int64_t ldx;        /* elements; multiple of 8 */
+    void* codes;        /* device, rows x cols bytes (I8, E4M3) or rows x cols/2 bytes (I4) */
+    void* codes_neg;    /* device or NULL, see above */
+    int64_t ld_codes;   /* bytes; multiple of 16 (8 for I4) */
+    float* scale;       /* device; input, or output when dynamic */
+    float* scale_neg;   /* device or NULL (required when dual) */
+    int64_t seg_rows;   /* rows per row segment; 0 means rows */
+    int64_t seg_stride;
+    int64_t row_stride;
+    int64_t kseg_stride;
+    int32_t n_kseg;     /* 1 .. SEGQ_MAX_KSEG */
+    int32_t dual;
+    uint32_t dual_kseg_mask;
+    int32_t dynamic;
+    int64_t kseg_bounds[SEGQ_MAX_KSEG + 1]; /* column segment i = [bounds[i], bounds[i+1]); multiples of 16 */
+} segq_quant_desc;
+
+int segq_quantize(const segq_quant_desc* d, segq_stream_t stream);
+
+/* The reference's two weight entry points under their own names
+ * (segquant/src/real_quant/seg_utils.h:82-119): one scale by value, or one per
+ * output row.  weights is (n, k) row-major contiguous; codes is (n, k) bytes,
+ * or n*k/2 bytes for int4. */
+int segq_quantize_weights_scalar(const void* weights, int32_t w_dtype, int64_t n, int64_t k,
+                                 void* codes, int32_t code_fmt, float scale_w, segq_stream_t stream);
+int segq_quantize_weights_rows(const void* weights, int32_t w_dtype, int64_t n, int64_t k,
+                               void* codes, int32_t code_fmt, const float* scale_w_rows,
+                               segq_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Segmented GEMM with fused de-quantisation and bias.
+ *
+ * Replaces, in one launch, the reference's GEMM launches and the de-quantise
+ * pass that follows them: launch_gemm_scaled / launch_batched_gemm_scaled /
+ * launch_array_gemm_scaled (segquant/src/real_quant/real_gemm.cu:424-532) and
+ * real_dequantize_scaled_kernel / real_dequantize_dual_scaled_kernel
+ * (segquant/src/real_quant/dequantizer.cuh:35-74), plus the recombination and
+ * bias add of SegmentLinear.forward (segquant/layers/SegmentLinear.py:233-241).
+ *
+ *   out[z][m][n] = sum over ranges r of
+ *                    ( sum_{k in r} A_r[z][m][k] * B[z][n][k] ) / (sx_r[z][m] * sw_r[z][n])
+ *                  + bias[n]
+ *
+ * A "range" is a run of contraction columns that shares one pair of scales:
+ * an input-channel segment, or one sign half of a DualScale segment.  Output-
+ * column segments need no range: they are a per-column sw vector.  A_r is
+ * chosen by a_sel:
+ *   0  the code tensor a
+ *   1  the second code tensor a_neg (the reference's Xn)
+ *   2  the non-negative codes of a, negatives read as zero  (merged DualScale)
+ *   3  the negative codes of a, the rest read as zero       (merged DualScale)
+ * Accumulation is int32 for integer codes and fp32 for e4m3; the partial sums
+ * of different ranges are combined in fp32 and rounded once to out_dtype.
+ * ---------------------------------------------------------------------- */
+typedef struct segq_krange {
+    int64_t k_begin;        /* first contraction column; multiple of 16 (32 with int4 weights) */
+    int64_t k_len;          /* multiple of 16 (32 with int4 weights) */
+    int32_t a_sel;
+    int32_t sx_row_stride;  /* 0: sx[0] for every row; 1: sx[m] */
+    int32_t sw_col_stride;  /* 0: sw[0] for every column; 1: sw[n] */
+    int32_t reserved;
+    const float* sx;        /* device */
+    const float* sw;        /* device */
+} segq_krange;
+
+typedef struct segq_gemm_desc {
+    int32_t a_fmt;      /* SEGQ_CODE_I8 | SEGQ_CODE_E4M3 */
+    int32_t b_fmt;      /* same as a_fmt, or SEGQ_CODE_I4 with a_fmt == SEGQ_CODE_I8 */
+    int32_t out_dtype;  /* segq_dtype; SEGQ_ACC needs n_ranges == 1 and ignores scales and bias */
+    int32_t bias_dtype; /* F32 | F16 | BF16 */
+    int64_t m, n;
+    const void* a;      /* device, m x K codes, row stride lda bytes (multiple of 16) */
+    const void* a_neg;  /* device or NULL */
+    int64_t lda;
+    const void* b;      /* device, n x K codes, row stride ldb bytes (multiple of 16); int4: K/2 bytes per row */
+    int64_t ldb;
+    void* out;          /* device, m x n, row stride ldo elements */
+    int64_t ldo;
+    const void* bias;   /* device, n entries, or NULL */
+    int64_t batch;      /* >= 1 independent problems (the reference's leading S dimension) */
+    int64_t batch_stride_a;   /* bytes */
+    int64_t batch_stride_b;   /* bytes */
+    int64_t batch_stride_out; /* elements */
+    int64_t batch_stride_sx;  /* floats, applied to every range's sx */
+    int64_t batch_stride_sw;  /* floats, applied to every range's sw */
+    int32_t n_ranges;   /* 1 .. SEGQ_MAX_RANGES */
+    int32_t tile;       /* 0 = choose; otherwise a tile configuration id, see segq_gemm_tile_count */
+    segq_krange ranges[SEGQ_MAX_RANGES];
+} segq_gemm_desc;
+
+int segq_gemm(const segq_gemm_desc* d, segq_stream_t stream);
+
+/* Number of tile configurations accepted in segq_gemm_desc.tile (ids 1..count). */
+int segq_gemm_tile_count(void);
+
+/* Quantise-then-multiply in one call: q writes its codes into a caller-provided
+ * workspace that g reads as its a (and a_neg).  Replaces the body of
+ * real_quantized_gemm_scaled / real_quantized_gemm_dual_scaled
+ * (segquant/src/real_quant/real_gemm.cu:643-894) without their temporaries,
+ * host synchronisation or per-call device allocation. */
+int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream);
+
+/* out[i] = float(e4m3(x[i])) in the dtype of x.  Replaces fake_e4m3fy
+ * (segquant/src/fake_quant/quantizer_fp8.cu:34-51). */
+int segq_fake_e4m3(const void* x, void* out, int32_t dtype, int64_t numel, segq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SEGQ_H */

@@ -1,0 +1,177 @@
+// C ABI of libsegq: argument checks, kernel selection, launches.
+#include "segq_gemm_kernel.h"
+#include <string.h>
+
+namespace segq {
+
+static thread_local char g_err[512] = "";
+
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SEGQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return SEGQ_OK;
+}
+
+int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value);
+int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipStream_t st);
+
+static bool is_float_dtype(int t) { return t == SEGQ_F32 || t == SEGQ_F16 || t == SEGQ_BF16; }
+static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Tile choice when the caller leaves it to the library: the largest tile that
+// still yields at least one workgroup per CU, preferring square tiles.
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold) {
+    const int order_plain[] = {0, 1, 4, 2, 3};
+    const int order_fold[] = {1, 4, 2, 3};
+    const int* order = fold ? order_fold : order_plain;
+    const int cnt = fold ? 4 : 5;
+    for (int i = 0; i < cnt; ++i) {
+        const TileCfg& c = TILE_CFGS[order[i]];
+        const int64_t tiles = ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
+        if (tiles >= 256) return order[i];
+    }
+    return 3;
+}
+
+static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
+    if (!d) return fail(SEGQ_ERR_ARG, "segq_gemm: null descriptor");
+    if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
+    if (d->m == 0 || d->n == 0) return SEGQ_OK;
+    if (d->m > 0x7fffffff / 2 || d->n > 0x7fffffff / 2) return fail(SEGQ_ERR_ARG, "segq_gemm: m or n too large");
+    if (!d->a || !d->b || !d->out) return fail(SEGQ_ERR_ARG, "segq_gemm: null a, b or out");
+    if (d->n_ranges < 1 || d->n_ranges > SEGQ_MAX_RANGES) return fail(SEGQ_ERR_ARG, "segq_gemm: n_ranges %d out of range", d->n_ranges);
+    const bool i8 = d->a_fmt == SEGQ_CODE_I8 && d->b_fmt == SEGQ_CODE_I8;
+    const bool f8 = d->a_fmt == SEGQ_CODE_E4M3 && d->b_fmt == SEGQ_CODE_E4M3;
+    const bool w4 = d->a_fmt == SEGQ_CODE_I8 && d->b_fmt == SEGQ_CODE_I4;
+    if (!i8 && !f8 && !w4) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: no kernel for a_fmt %d with b_fmt %d", d->a_fmt, d->b_fmt);
+    if (d->out_dtype != SEGQ_ACC && !is_float_dtype(d->out_dtype)) return fail(SEGQ_ERR_ARG, "segq_gemm: bad out_dtype %d", d->out_dtype);
+    if (d->bias && !is_float_dtype(d->bias_dtype)) return fail(SEGQ_ERR_ARG, "segq_gemm: bad bias_dtype %d", d->bias_dtype);
+    if (d->out_dtype == SEGQ_ACC && d->n_ranges != 1) return fail(SEGQ_ERR_ARG, "segq_gemm: raw accumulators need exactly one range");
+    if (d->lda % 16 || d->ldb % 16 || !al(d->a, 16) || !al(d->b, 16) || (d->a_neg && !al(d->a_neg, 16)) ||
+        d->batch_stride_a % 16 || d->batch_stride_b % 16)
+        return fail(SEGQ_ERR_ARG, "segq_gemm: a and b need 16-byte aligned bases and row strides");
+    if (d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
+
+    GemmParams p;
+    memset(&p, 0, sizeof(p));
+    const int64_t kalign = w4 ? 32 : 16;
+    int64_t kmax = 0, ktotal = 0;
+    for (int i = 0; i < d->n_ranges; ++i) {
+        const segq_krange& r = d->ranges[i];
+        // the K rule of the reference's GEMM (segquant/src/real_quant/real_gemm.cu:237-247)
+        if (r.k_begin < 0 || r.k_len <= 0 || r.k_begin % kalign || r.k_len % kalign)
+            return fail(SEGQ_ERR_ARG, "segq_gemm: range %d: k_begin %lld and k_len %lld must be positive multiples of %lld",
+                        i, (long long)r.k_begin, (long long)r.k_len, (long long)kalign);
+        if (r.a_sel < 0 || r.a_sel > 3) return fail(SEGQ_ERR_ARG, "segq_gemm: range %d: bad a_sel %d", i, r.a_sel);
+        if (r.a_sel == 1 && !d->a_neg) return fail(SEGQ_ERR_ARG, "segq_gemm: range %d reads a_neg, which is null", i);
+        if (d->out_dtype != SEGQ_ACC && (!r.sx || !r.sw)) return fail(SEGQ_ERR_ARG, "segq_gemm: range %d has a null scale", i);
+        if ((r.sx_row_stride | 1) != 1 || (r.sw_col_stride | 1) != 1) return fail(SEGQ_ERR_ARG, "segq_gemm: range %d: scale strides are 0 or 1", i);
+        KRange& o = p.r[i];
+        o.k0 = (int32_t)r.k_begin;
+        o.k1 = (int32_t)(r.k_begin + r.k_len);
+        o.a_sel = r.a_sel;
+        o.sx_rs = r.sx_row_stride;
+        o.sw_cs = r.sw_col_stride;
+        o.sx = r.sx;
+        o.sw = r.sw;
+        if (r.k_begin + r.k_len > kmax) kmax = r.k_begin + r.k_len;
+        ktotal += r.k_len;
+    }
+    if (kmax > d->lda || (w4 ? (kmax / 2 > d->ldb) : (kmax > d->ldb)))
+        return fail(SEGQ_ERR_ARG, "segq_gemm: a range ends at %lld, beyond the row stride", (long long)kmax);
+    // int4 weights are staged as value*16: keep |acc| below 2^31
+    if (w4 && ktotal > 131071) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: K too large for int4 weights");
+    if (kmax > 0x7fffff00) return fail(SEGQ_ERR_ARG, "segq_gemm: K too large");
+
+    p.A = static_cast<const uint8_t*>(d->a);
+    p.A2 = static_cast<const uint8_t*>(d->a_neg);
+    p.B = static_cast<const uint8_t*>(d->b);
+    p.C = d->out;
+    p.bias = d->out_dtype == SEGQ_ACC ? nullptr : d->bias;
+    p.M = (int32_t)d->m;
+    p.N = (int32_t)d->n;
+    p.lda = d->lda; p.ldb = d->ldb; p.ldc = d->ldo;
+    p.bsA = d->batch_stride_a; p.bsB = d->batch_stride_b; p.bsC = d->batch_stride_out;
+    p.bsSx = d->batch_stride_sx; p.bsSw = d->batch_stride_sw;
+    p.out_dtype = d->out_dtype; p.bias_dtype = d->bias_dtype;
+    p.nr = d->n_ranges;
+    const bool fold = d->n_ranges > 1;
+    int cfg;
+    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold);
+    else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
+    else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
+    const TileCfg& c = TILE_CFGS[cfg];
+    p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);
+    p.tiles_n = (int32_t)((d->n + c.bn - 1) / c.bn);
+    p.group_m = 8;
+    if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff || d->batch > 65535) return fail(SEGQ_ERR_ARG, "segq_gemm: grid too large");
+    const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
+    p.vec_store = ((d->ldo * osz) % (4 * osz) == 0) && ((d->batch_stride_out * osz) % (4 * osz) == 0) && al(d->out, 4 * osz);
+    if (i8) return launch_gemm_i8(p, cfg, fold, d->batch, st);
+    if (f8) return launch_gemm_f8(p, cfg, fold, d->batch, st);
+    return launch_gemm_w4(p, cfg, fold, d->batch, st);
+}
+
+}  // namespace segq
+
+using namespace segq;
+
+extern "C" {
+
+int segq_version(void) { return 100; }
+
+const char* segq_last_error(void) { return g_err; }
+
+int segq_quantize(const segq_quant_desc* d, segq_stream_t stream) {
+    return quantize_impl(d, static_cast<hipStream_t>(stream), nullptr);
+}
+
+static void weight_desc(segq_quant_desc* q, const void* w, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t fmt) {
+    memset(q, 0, sizeof(*q));
+    q->x = w; q->x_dtype = w_dtype; q->code_fmt = fmt;
+    q->rows = n; q->cols = k; q->ldx = k;
+    q->codes = codes; q->ld_codes = fmt == SEGQ_CODE_I4 ? k / 2 : k;
+    q->n_kseg = 1;
+}
+
+int segq_quantize_weights_scalar(const void* weights, int32_t w_dtype, int64_t n, int64_t k, void* codes,
+                                 int32_t code_fmt, float scale_w, segq_stream_t stream) {
+    segq_quant_desc q;
+    weight_desc(&q, weights, w_dtype, n, k, codes, code_fmt);
+    return quantize_impl(&q, static_cast<hipStream_t>(stream), &scale_w);
+}
+
+int segq_quantize_weights_rows(const void* weights, int32_t w_dtype, int64_t n, int64_t k, void* codes,
+                               int32_t code_fmt, const float* scale_w_rows, segq_stream_t stream) {
+    segq_quant_desc q;
+    weight_desc(&q, weights, w_dtype, n, k, codes, code_fmt);
+    q.scale = const_cast<float*>(scale_w_rows);
+    q.row_stride = 1;
+    return quantize_impl(&q, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int segq_gemm(const segq_gemm_desc* d, segq_stream_t stream) { return gemm_impl(d, static_cast<hipStream_t>(stream)); }
+
+int segq_gemm_tile_count(void) { return NUM_TILE_CFG; }
+
+int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream) {
+    if (!q || !g) return fail(SEGQ_ERR_ARG, "segq_linear: null descriptor");
+    if (q->codes != g->a) return fail(SEGQ_ERR_ARG, "segq_linear: the GEMM must read the codes the quantise step writes");
+    const int rc = quantize_impl(q, static_cast<hipStream_t>(stream), nullptr);
+    if (rc != SEGQ_OK) return rc;
+    return gemm_impl(g, static_cast<hipStream_t>(stream));
+}
+
+int segq_fake_e4m3(const void* x, void* out, int32_t dtype, int64_t numel, segq_stream_t stream) {
+    return fake_e4m3_impl(x, out, dtype, numel, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,40 @@
+// Shared host/device helpers of libsegq (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "segq.h"
+
+namespace segq {
+
+// Records a message for segq_last_error() and returns the status, so callers
+// can write `return fail(SEGQ_ERR_ARG, "...")`.
+int fail(int status, const char* fmt, ...);
+
+// Checks the launch that was just enqueued.
+int check_launch(const char* what);
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    return u >> 16;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
+}
+
+}  // namespace segq

@@ -1,0 +1,367 @@
+// Quantise kernels of libsegq: float matrix -> int8 / e4m3 / packed-int4 codes.
+//
+// One pass over HBM: every thread converts runs of 16 consecutive elements of a
+// row (two or four 16-byte loads, one 16-byte or 8-byte store).  The static
+// kernel is a flat grid over such runs; the dynamic kernel gives a row to a
+// block, keeps the row in registers while it reduces the absolute maximum, and
+// quantises from registers.
+#include "segq_common.h"
+
+namespace segq {
+
+struct QuantParams {
+    const void* x;
+    void* codes;
+    void* codes_neg;
+    float* scale;
+    float* scale_neg;
+    int64_t rows, cols, ldx, ldc;
+    int64_t seg_rows, seg_stride, row_stride, kseg_stride;
+    int32_t x_dtype, fmt;
+    int32_t n_kseg, dual, dynamic;
+    uint32_t dual_mask;
+    float scale_imm;  // used when scale == nullptr (one scale passed by value)
+    int32_t kb[SEGQ_MAX_KSEG + 1];
+};
+
+// ---- element conversion --------------------------------------------------
+
+// 16 consecutive elements of dtype DT starting at p (16-byte aligned) -> fp32.
+template <int DT>
+__device__ __forceinline__ void load16(const void* p, float (&v)[16]) {
+    if constexpr (DT == SEGQ_F32) {
+        const float4* q = reinterpret_cast<const float4*>(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float4 t = q[i];
+            v[4 * i + 0] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* q = reinterpret_cast<const uint4*>(p);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint4 t = q[i];
+            uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (DT == SEGQ_BF16) {
+                    v[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
+                    v[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                } else {
+                    v[8 * i + 2 * j + 0] = f16_bits_to_f32(w[j] & 0xffffu);
+                    v[8 * i + 2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+                }
+            }
+        }
+    }
+}
+
+// clamp first, then round half to even; a NaN operand is dropped by fmaxf and
+// becomes the lower bound (segquant/src/real_quant/quantizer.cuh:31-35).
+__device__ __forceinline__ int q_i8(float v) { return (int)rintf(fminf(fmaxf(v, -128.0f), 127.0f)); }
+__device__ __forceinline__ int q_i4(float v) { return (int)rintf(fminf(fmaxf(v, -8.0f), 7.0f)); }
+
+// e4m3 with saturation to +-448 (fminf/fmaxf drop a NaN operand, so NaN is
+// patched afterwards: it encodes as 0x7F whatever its sign).
+__device__ __forceinline__ float sat_e4m3(float v) { return fminf(fmaxf(v, -448.0f), 448.0f); }
+
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(sat_e4m3(a), sat_e4m3(b), 0, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(sat_e4m3(c), sat_e4m3(d), r, true);
+    const uint32_t nan = (a != a ? 0xFFu : 0u) | (b != b ? 0xFF00u : 0u) | (c != c ? 0xFF0000u : 0u) |
+                         (d != d ? 0xFF000000u : 0u);
+    return ((uint32_t)r & ~nan) | (0x7F7F7F7Fu & nan);
+}
+
+__device__ __forceinline__ uint32_t pack4_i8(float a, float b, float c, float d) {
+    return (uint32_t)(q_i8(a) & 0xff) | ((uint32_t)(q_i8(b) & 0xff) << 8) |
+           ((uint32_t)(q_i8(c) & 0xff) << 16) | ((uint32_t)(q_i8(d) & 0xff) << 24);
+}
+
+// 8 values -> 8 nibbles, element 0 in the lowest nibble.
+__device__ __forceinline__ uint32_t pack8_i4(const float* v) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r |= (uint32_t)(q_i4(v[i]) & 0xf) << (4 * i);
+    return r;
+}
+
+// Encodes 16 scaled values and stores them at row-relative element offset col.
+template <int FMT>
+__device__ __forceinline__ void store16(void* row_base, int64_t col, const float (&v)[16]) {
+    if constexpr (FMT == SEGQ_CODE_I4) {
+        uint2 o;
+        o.x = pack8_i4(v);
+        o.y = pack8_i4(v + 8);
+        *reinterpret_cast<uint2*>(static_cast<uint8_t*>(row_base) + (col >> 1)) = o;
+    } else {
+        uint4 o;
+        if constexpr (FMT == SEGQ_CODE_I8) {
+            o.x = pack4_i8(v[0], v[1], v[2], v[3]);
+            o.y = pack4_i8(v[4], v[5], v[6], v[7]);
+            o.z = pack4_i8(v[8], v[9], v[10], v[11]);
+            o.w = pack4_i8(v[12], v[13], v[14], v[15]);
+        } else {
+            o.x = pack4_e4m3(v[0], v[1], v[2], v[3]);
+            o.y = pack4_e4m3(v[4], v[5], v[6], v[7]);
+            o.z = pack4_e4m3(v[8], v[9], v[10], v[11]);
+            o.w = pack4_e4m3(v[12], v[13], v[14], v[15]);
+        }
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(row_base) + col) = o;
+    }
+}
+
+// Scales 16 raw values and writes the merged tensor, or Xp and Xn.
+template <int FMT>
+__device__ __forceinline__ void encode16(const QuantParams& p, int64_t row, int64_t col, const float (&x)[16],
+                                         float s_pos, float s_neg, bool two_tensors) {
+    const int64_t cstride = p.ldc;
+    uint8_t* base = static_cast<uint8_t*>(p.codes) + row * cstride;
+    float v[16];
+    if (!two_tensors) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = x[i] * ((x[i] >= 0.0f) ? s_pos : s_neg);
+        store16<FMT>(base, col, v);
+    } else {
+        // The branch that was not taken holds code(0) (quantizer.cuh:193-203).
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = (x[i] >= 0.0f) ? x[i] * s_pos : 0.0f;
+        store16<FMT>(base, col, v);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = (x[i] >= 0.0f) ? 0.0f : x[i] * s_neg;
+        store16<FMT>(static_cast<uint8_t*>(p.codes_neg) + row * cstride, col, v);
+    }
+}
+
+__device__ __forceinline__ int64_t row_scale_index(const QuantParams& p, int64_t row) {
+    if (p.seg_rows >= p.rows) return row * p.row_stride;
+    const int64_t seg = row / p.seg_rows;
+    return seg * p.seg_stride + (row - seg * p.seg_rows) * p.row_stride;
+}
+
+__device__ __forceinline__ int kseg_of(const QuantParams& p, int col) {
+    int s = 0;
+    for (int i = 1; i < p.n_kseg; ++i) s += (col >= p.kb[i]) ? 1 : 0;
+    return s;
+}
+
+// ---- static scales ---------------------------------------------------------
+template <int DT, int FMT>
+__global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) {
+    const int64_t cpr = p.cols >> 4;  // runs of 16 per row
+    const int64_t run = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (run >= p.rows * cpr) return;
+    const int64_t row = run / cpr;
+    const int col = (int)(run - row * cpr) << 4;
+    const int ks = kseg_of(p, col);
+    const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
+    const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
+    const float s_pos = p.scale ? p.scale[si] : p.scale_imm;
+    const float s_neg = dual ? p.scale_neg[si] : s_pos;
+    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+    float x[16];
+    load16<DT>(static_cast<const uint8_t*>(p.x) + (row * p.ldx + col) * esz, x);
+    encode16<FMT>(p, row, col, x, s_pos, s_neg, p.dual && p.codes_neg != nullptr);
+}
+
+// ---- dynamic per-row scales ------------------------------------------------
+__device__ __forceinline__ float block_max(float v, float* red) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    const int w = threadIdx.x >> 6;
+    __syncthreads();  // red may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+template <int FMT>
+__device__ __forceinline__ float qmax_pos() {
+    return FMT == SEGQ_CODE_I8 ? 127.0f : (FMT == SEGQ_CODE_I4 ? 7.0f : 448.0f);
+}
+template <int FMT>
+__device__ __forceinline__ float qmax_neg() {
+    return FMT == SEGQ_CODE_I8 ? 128.0f : (FMT == SEGQ_CODE_I4 ? 8.0f : 448.0f);
+}
+
+// One block per row.  Up to CACHE runs per thread stay in registers between the
+// reduction and the encode; longer rows are read again (they hit in L2).
+template <int DT, int FMT>
+__global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p) {
+    constexpr int CACHE = 4;
+    __shared__ float red_a[4];
+    __shared__ float red_b[4];
+    const int64_t row = blockIdx.x;
+    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+    const uint8_t* xrow = static_cast<const uint8_t*>(p.x) + row * p.ldx * esz;
+    const float eps = 5.9604644775390625e-08f;  // 2^-24
+    const bool two = p.dual && p.codes_neg != nullptr;
+    for (int ks = 0; ks < p.n_kseg; ++ks) {
+        const int c0 = p.kb[ks] >> 4, c1 = p.kb[ks + 1] >> 4;
+        const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
+        float cache[CACHE][16];
+        float amax_p = 0.0f, amax_n = 0.0f;
+#pragma unroll
+        for (int i = 0; i < CACHE; ++i) {
+            const int c = c0 + threadIdx.x + i * 256;
+            if (c < c1) {
+                load16<DT>(xrow + (size_t)c * 16 * esz, cache[i]);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float a = cache[i][j];
+                    // strict masks: x > 0 and x < 0 (quantizer.py:172-189); NaN is ignored
+                    amax_p = fmaxf(amax_p, a > 0.0f ? a : 0.0f);
+                    amax_n = fmaxf(amax_n, a < 0.0f ? -a : 0.0f);
+                }
+            }
+        }
+        for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
+            float t[16];
+            load16<DT>(xrow + (size_t)c * 16 * esz, t);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                amax_p = fmaxf(amax_p, t[j] > 0.0f ? t[j] : 0.0f);
+                amax_n = fmaxf(amax_n, t[j] < 0.0f ? -t[j] : 0.0f);
+            }
+        }
+        amax_p = block_max(amax_p, red_a);
+        amax_n = block_max(amax_n, red_b);
+        float s_pos, s_neg;
+        if (dual) {
+            s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
+            s_neg = qmax_neg<FMT>() / fmaxf(amax_n, eps);
+        } else {
+            s_pos = s_neg = qmax_pos<FMT>() / fmaxf(fmaxf(amax_p, amax_n), eps);
+        }
+        const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
+        if (threadIdx.x == 0) {
+            p.scale[si] = s_pos;
+            if (p.dual) p.scale_neg[si] = s_neg;
+        }
+#pragma unroll
+        for (int i = 0; i < CACHE; ++i) {
+            const int c = c0 + threadIdx.x + i * 256;
+            if (c < c1) encode16<FMT>(p, row, (int64_t)c << 4, cache[i], s_pos, s_neg, two);
+        }
+        for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
+            float t[16];
+            load16<DT>(xrow + (size_t)c * 16 * esz, t);
+            encode16<FMT>(p, row, (int64_t)c << 4, t, s_pos, s_neg, two);
+        }
+    }
+}
+
+// ---- fake e4m3 round trip ----------------------------------------------------
+__device__ __forceinline__ float e4m3_roundtrip(float v) {
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(sat_e4m3(v), 0.0f, 0, false);
+    return (v != v) ? v : __builtin_amdgcn_cvt_f32_fp8(r, 0);
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) fake_e4m3_kernel(const void* x, void* out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    if constexpr (DT == SEGQ_F32) {
+        static_cast<float*>(out)[i] = e4m3_roundtrip(static_cast<const float*>(x)[i]);
+    } else if constexpr (DT == SEGQ_BF16) {
+        const float v = bf16_bits_to_f32(static_cast<const uint16_t*>(x)[i]);
+        static_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(e4m3_roundtrip(v));
+    } else {
+        const float v = f16_bits_to_f32(static_cast<const uint16_t*>(x)[i]);
+        static_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_f16_bits(e4m3_roundtrip(v));
+    }
+}
+
+// ---- host side ---------------------------------------------------------------
+template <int DT, int FMT>
+static int launch_quant(const QuantParams& p, hipStream_t st) {
+    if (p.dynamic) {
+        hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT>), dim3((unsigned)p.rows), dim3(256), 0, st, p);
+    } else {
+        const int64_t runs = p.rows * (p.cols >> 4);
+        hipLaunchKernelGGL((quant_static_kernel<DT, FMT>), dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, st, p);
+    }
+    return check_launch("segq_quantize");
+}
+
+template <int DT>
+static int launch_quant_fmt(const QuantParams& p, hipStream_t st) {
+    switch (p.fmt) {
+        case SEGQ_CODE_I8: return launch_quant<DT, SEGQ_CODE_I8>(p, st);
+        case SEGQ_CODE_E4M3: return launch_quant<DT, SEGQ_CODE_E4M3>(p, st);
+        case SEGQ_CODE_I4: return launch_quant<DT, SEGQ_CODE_I4>(p, st);
+    }
+    return fail(SEGQ_ERR_ARG, "segq_quantize: unknown code_fmt %d", p.fmt);
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value) {
+    if (!d) return fail(SEGQ_ERR_ARG, "segq_quantize: null descriptor");
+    if (d->rows < 0 || d->cols < 0) return fail(SEGQ_ERR_ARG, "segq_quantize: negative size");
+    if (d->rows == 0 || d->cols == 0) return SEGQ_OK;
+    if (!d->x || !d->codes || (!d->scale && !scale_by_value))
+        return fail(SEGQ_ERR_ARG, "segq_quantize: null x, codes or scale");
+    if (scale_by_value && (d->dual || d->dynamic))
+        return fail(SEGQ_ERR_ARG, "segq_quantize: a scale by value is static and single");
+    if (d->cols % 16) return fail(SEGQ_ERR_ARG, "segq_quantize: cols (%lld) must be a multiple of 16", (long long)d->cols);
+    if (d->x_dtype != SEGQ_F32 && d->x_dtype != SEGQ_F16 && d->x_dtype != SEGQ_BF16)
+        return fail(SEGQ_ERR_ARG, "segq_quantize: x_dtype %d is not a float type", d->x_dtype);
+    const int64_t esz = d->x_dtype == SEGQ_F32 ? 4 : 2;
+    if (d->ldx < d->cols || (d->ldx * esz) % 16) return fail(SEGQ_ERR_ARG, "segq_quantize: ldx must be >= cols and 16-byte aligned");
+    const int64_t min_ldc = d->code_fmt == SEGQ_CODE_I4 ? d->cols / 2 : d->cols;
+    const int64_t ldc_align = d->code_fmt == SEGQ_CODE_I4 ? 8 : 16;
+    if (d->ld_codes < min_ldc || d->ld_codes % ldc_align) return fail(SEGQ_ERR_ARG, "segq_quantize: bad ld_codes %lld", (long long)d->ld_codes);
+    if (!aligned16(d->x) || (reinterpret_cast<uintptr_t>(d->codes) % ldc_align) ||
+        (d->codes_neg && (reinterpret_cast<uintptr_t>(d->codes_neg) % ldc_align)))
+        return fail(SEGQ_ERR_ARG, "segq_quantize: x and codes must be 16-byte aligned");
+    if (d->dual && !d->scale_neg) return fail(SEGQ_ERR_ARG, "segq_quantize: dual needs scale_neg");
+    if (d->n_kseg < 1 || d->n_kseg > SEGQ_MAX_KSEG) return fail(SEGQ_ERR_ARG, "segq_quantize: n_kseg %d out of range", d->n_kseg);
+    if (d->rows * (d->cols / 16) > (int64_t)0x7fffffff * 256 || d->cols > 0x7fffffff || d->rows > 0x7fffffff)
+        return fail(SEGQ_ERR_ARG, "segq_quantize: matrix too large");
+
+    QuantParams p{};
+    p.x = d->x; p.codes = d->codes; p.codes_neg = d->codes_neg;
+    p.scale = d->scale; p.scale_neg = d->scale_neg;
+    p.rows = d->rows; p.cols = d->cols; p.ldx = d->ldx; p.ldc = d->ld_codes;
+    p.seg_rows = d->seg_rows > 0 ? d->seg_rows : d->rows;
+    p.seg_stride = d->seg_stride; p.row_stride = d->row_stride; p.kseg_stride = d->kseg_stride;
+    p.x_dtype = d->x_dtype; p.fmt = d->code_fmt;
+    p.n_kseg = d->n_kseg; p.dual = d->dual ? 1 : 0; p.dynamic = d->dynamic ? 1 : 0;
+    p.dual_mask = d->dual_kseg_mask;
+    p.scale_imm = scale_by_value ? *scale_by_value : 0.0f;
+    if (d->n_kseg == 1) {
+        p.kb[0] = 0; p.kb[1] = (int32_t)d->cols;
+    } else {
+        if (d->kseg_bounds[0] != 0 || d->kseg_bounds[d->n_kseg] != d->cols)
+            return fail(SEGQ_ERR_ARG, "segq_quantize: kseg_bounds must span [0, cols]");
+        for (int i = 0; i <= d->n_kseg; ++i) {
+            if (d->kseg_bounds[i] % 16 || (i && d->kseg_bounds[i] <= d->kseg_bounds[i - 1]))
+                return fail(SEGQ_ERR_ARG, "segq_quantize: kseg_bounds must be increasing multiples of 16");
+            p.kb[i] = (int32_t)d->kseg_bounds[i];
+        }
+    }
+    if (p.dynamic && p.row_stride != 1 && p.rows != 1 && p.seg_rows != 1)
+        return fail(SEGQ_ERR_ARG, "segq_quantize: dynamic scales are per row (row_stride must be 1)");
+    switch (d->x_dtype) {
+        case SEGQ_F32: return launch_quant_fmt<SEGQ_F32>(p, st);
+        case SEGQ_F16: return launch_quant_fmt<SEGQ_F16>(p, st);
+        default: return launch_quant_fmt<SEGQ_BF16>(p, st);
+    }
+}
+
+int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipStream_t st) {
+    if (numel < 0) return fail(SEGQ_ERR_ARG, "segq_fake_e4m3: negative numel");
+    if (numel == 0) return SEGQ_OK;
+    if (!x || !out) return fail(SEGQ_ERR_ARG, "segq_fake_e4m3: null pointer");
+    const dim3 grid((unsigned)((numel + 255) / 256)), block(256);
+    switch (dtype) {
+        case SEGQ_F32: hipLaunchKernelGGL(fake_e4m3_kernel<SEGQ_F32>, grid, block, 0, st, x, out, numel); break;
+        case SEGQ_F16: hipLaunchKernelGGL(fake_e4m3_kernel<SEGQ_F16>, grid, block, 0, st, x, out, numel); break;
+        case SEGQ_BF16: hipLaunchKernelGGL(fake_e4m3_kernel<SEGQ_BF16>, grid, block, 0, st, x, out, numel); break;
+        default: return fail(SEGQ_ERR_ARG, "segq_fake_e4m3: dtype %d is not a float type", dtype);
+    }
+    return check_launch("segq_fake_e4m3");
+}
+
+}  // namespace segq

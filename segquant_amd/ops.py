@@ -1,0 +1,295 @@
+"""torch-facing wrappers over the C ABI of libsegq.
+
+torch is plumbing here: it owns device memory and the current stream.  Every
+function takes CUDA (ROCm) tensors, allocates outputs with torch, hands raw
+pointers to the library and raises ``RuntimeError`` on a non-zero status, which
+is what the reference's pybind functions do (segquant/src/real_quant/seg_utils.h).
+
+Two layers:
+
+* :func:`quantize` and :func:`gemm` expose the library's own, richer interface
+  (column segments, ranges, merged DualScale codes, fused bias).
+* :func:`real_quantized_gemm_scaled`, :func:`real_quantized_gemm_dual_scaled`,
+  :func:`real_quantized_quantize_weights` and :func:`fake_e4m3fy` keep the
+  reference's tensor contract (segquant/src/real_quant/real_gemm.cu:643-894,
+  :538-638; segquant/src/fake_quant/quantizer_fp8.cpp:25-39).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib as L
+
+FMT_INT8 = "int8"
+FMT_INT4 = "int4"
+FMT_E4M3 = "fpe4m3"
+
+_CODE = {FMT_INT8: L.CODE_I8, FMT_E4M3: L.CODE_E4M3, FMT_INT4: L.CODE_I4}
+_DTYPE = {torch.float32: L.F32, torch.float16: L.F16, torch.bfloat16: L.BF16}
+
+
+def _dt(t: torch.dtype) -> int:
+    try:
+        return _DTYPE[t]
+    except KeyError:
+        raise RuntimeError(f"unsupported float dtype {t}") from None
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("libsegq needs tensors on the GPU")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def code_dtype(fmt: str) -> torch.dtype:
+    """Storage dtype of codes: int8 as int8, e4m3 and packed int4 as uint8
+    (segquant/src/real_quant/seg_utils.h:25-45)."""
+    return torch.int8 if fmt == FMT_INT8 else torch.uint8
+
+
+# ---------------------------------------------------------------------------
+# quantise
+# ---------------------------------------------------------------------------
+def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional[torch.Tensor] = None, *,
+             seg_rows: int = 0, seg_stride: int = 0, row_stride: int = 0,
+             kseg_bounds: Optional[Sequence[int]] = None, kseg_stride: int = 0,
+             dual: bool = False, dual_kseg_mask: int = 0xFFFFFFFF, dynamic: bool = False,
+             two_tensors: bool = False, out: Optional[torch.Tensor] = None,
+             out_neg: Optional[torch.Tensor] = None):
+    """Quantise a 2-D float matrix ``x`` (rows, cols) to codes.
+
+    See ``segq_quantize`` in include/segq.h for the scale indexing.  Returns the
+    code tensor, or ``(Xp, Xn)`` when ``two_tensors`` (DualScale in the
+    reference's two-tensor layout).  With ``dynamic`` the scale tensors are
+    written by the kernel.
+    """
+    _need_cuda(x, scale, scale_neg)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("quantize expects a 2-D tensor with a contiguous last dimension")
+    rows, cols = x.shape
+    ccols = cols // 2 if fmt == FMT_INT4 else cols
+    if out is None:
+        out = torch.empty((rows, ccols), dtype=code_dtype(fmt), device=x.device)
+    if two_tensors and out_neg is None:
+        out_neg = torch.empty_like(out)
+    d = L.QuantDesc()
+    d.x = x.data_ptr(); d.x_dtype = _dt(x.dtype); d.code_fmt = _CODE[fmt]
+    d.rows = rows; d.cols = cols; d.ldx = x.stride(0) if rows > 1 else cols
+    d.codes = out.data_ptr(); d.codes_neg = out_neg.data_ptr() if two_tensors else None
+    d.ld_codes = out.stride(0) if rows > 1 else ccols
+    if scale.dtype != torch.float32 or (scale_neg is not None and scale_neg.dtype != torch.float32):
+        raise RuntimeError("scales must be float32")
+    d.scale = scale.data_ptr(); d.scale_neg = scale_neg.data_ptr() if scale_neg is not None else None
+    d.seg_rows = seg_rows; d.seg_stride = seg_stride; d.row_stride = row_stride; d.kseg_stride = kseg_stride
+    if kseg_bounds is None:
+        d.n_kseg = 1
+    else:
+        d.n_kseg = len(kseg_bounds) - 1
+        if d.n_kseg > L.SEGQ_MAX_KSEG:
+            raise RuntimeError(f"at most {L.SEGQ_MAX_KSEG} column segments")
+        for i, b in enumerate(kseg_bounds):
+            d.kseg_bounds[i] = int(b)
+    d.dual = 1 if dual else 0; d.dual_kseg_mask = dual_kseg_mask & 0xFFFFFFFF; d.dynamic = 1 if dynamic else 0
+    L.check(L.lib().segq_quantize(C.byref(d), _stream()))
+    return (out, out_neg) if two_tensors else out
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+@dataclass
+class Range:
+    """A run of contraction columns sharing one (sx, sw) pair; see segq_krange."""
+    k_begin: int
+    k_len: int
+    sx: Optional[torch.Tensor]
+    sw: Optional[torch.Tensor]
+    a_sel: int = 0
+    sx_row_stride: int = 0
+    sw_col_stride: int = 0
+
+
+def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
+         out_dtype, lda: int, ldb: int, a_neg: Optional[torch.Tensor] = None,
+         bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
+         batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
+         tile: int = 0) -> torch.Tensor:
+    """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
+
+    ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
+    accumulators (int32 for integer codes, float32 for e4m3).
+    """
+    _need_cuda(a, b, a_neg, bias)
+    raw = out_dtype == "acc"
+    if raw:
+        tdt = torch.float32 if a_fmt == FMT_E4M3 else torch.int32
+    else:
+        tdt = out_dtype
+    if out is None:
+        out = torch.empty((batch, m, n) if batch > 1 else (m, n), dtype=tdt, device=a.device)
+    d = L.GemmDesc()
+    d.a_fmt = _CODE[a_fmt]; d.b_fmt = _CODE[b_fmt]
+    d.out_dtype = L.ACC if raw else _dt(tdt)
+    d.m = m; d.n = n
+    d.a = a.data_ptr(); d.a_neg = a_neg.data_ptr() if a_neg is not None else None; d.lda = lda
+    d.b = b.data_ptr(); d.ldb = ldb
+    d.out = out.data_ptr(); d.ldo = n
+    if bias is not None:
+        if bias.numel() != n or not bias.is_contiguous():
+            raise RuntimeError("bias must be a contiguous vector with one entry per output column")
+        d.bias = bias.data_ptr(); d.bias_dtype = _dt(bias.dtype)
+    d.batch = batch; d.batch_stride_a = batch_stride_a; d.batch_stride_b = batch_stride_b
+    d.batch_stride_out = m * n; d.batch_stride_sx = batch_stride_sx; d.batch_stride_sw = batch_stride_sw
+    if not 1 <= len(ranges) <= L.SEGQ_MAX_RANGES:
+        raise RuntimeError(f"1..{L.SEGQ_MAX_RANGES} ranges")
+    d.n_ranges = len(ranges); d.tile = tile
+    for i, r in enumerate(ranges):
+        kr = d.ranges[i]
+        kr.k_begin = r.k_begin; kr.k_len = r.k_len; kr.a_sel = r.a_sel
+        kr.sx_row_stride = r.sx_row_stride; kr.sw_col_stride = r.sw_col_stride
+        _need_cuda(r.sx, r.sw)
+        for s in (r.sx, r.sw):
+            if s is not None and s.dtype != torch.float32:
+                raise RuntimeError("scales must be float32")
+        kr.sx = r.sx.data_ptr() if r.sx is not None else None
+        kr.sw = r.sw.data_ptr() if r.sw is not None else None
+    L.check(L.lib().segq_gemm(C.byref(d), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# the reference's tensor contract
+# ---------------------------------------------------------------------------
+def _shapes(inputs: torch.Tensor, weights: torch.Tensor, fmt_w: str):
+    S = inputs.shape[0]
+    K = inputs.shape[-1]
+    M = 1
+    for d in inputs.shape[1:-1]:
+        M *= d
+    if weights.shape[0] != S:
+        raise RuntimeError("inputs and weights must have the same number of segments")
+    if fmt_w == FMT_INT4:
+        N = weights.shape[1] * 2 // K  # segquant/src/real_quant/real_gemm.cu:670
+        if weights.dim() != 2 or N * K != weights.shape[1] * 2:
+            raise RuntimeError("int4 weights must be (segments, N*K/2) bytes")
+    else:
+        if weights.dim() != 3 or weights.shape[2] != K:
+            raise RuntimeError("weights must be (segments, N, K)")
+        N = weights.shape[1]
+    return S, M, N, K
+
+
+def _check_contract(inputs, weights, fmt_w, *scales):
+    _need_cuda(inputs, weights, *scales)
+    if not inputs.is_contiguous() or not weights.is_contiguous():
+        raise RuntimeError("tensor must be contiguous")
+    if weights.dtype != code_dtype(fmt_w):
+        raise RuntimeError("tensor dtype failed")
+    for s in scales:
+        if s.dtype != torch.float32 or not s.is_contiguous():
+            raise RuntimeError("scales must be contiguous float32")
+
+
+def real_quantized_gemm_scaled(fmt_a: str, fmt_w: str, inputs: torch.Tensor, weights: torch.Tensor,
+                               scale_x: torch.Tensor, scale_w: torch.Tensor) -> torch.Tensor:
+    """``<prefix>_real_quantized_gemm_scaled`` (segquant/src/real_quant/real_gemm.cu:643-750).
+
+    inputs (S, ..., M, K) float; weights (S, N, K) codes or (S, N*K/2) bytes for
+    int4; scale_x has S or S*M entries, scale_w S or S*N; returns a new
+    (S, ..., M, N) tensor in ``inputs.dtype``.  One quantise launch over all S
+    segments and one batched GEMM launch; no temporaries beyond the codes.
+    """
+    _check_contract(inputs, weights, fmt_w, scale_x, scale_w)
+    S, M, N, K = _shapes(inputs, weights, fmt_w)
+    per_seg_x = scale_x.numel() == S
+    per_seg_w = scale_w.numel() == S
+    if not per_seg_x and scale_x.numel() != S * M:
+        raise RuntimeError(f"scale_x has {scale_x.numel()} entries, expected {S} or {S * M}")
+    if not per_seg_w and scale_w.numel() != S * N:
+        raise RuntimeError(f"scale_w has {scale_w.numel()} entries, expected {S} or {S * N}")
+    codes = quantize(inputs.view(S * M, K), fmt_a, scale_x, seg_rows=M,
+                     seg_stride=1 if per_seg_x else M, row_stride=0 if per_seg_x else 1)
+    out = torch.empty((*inputs.shape[:-1], N), dtype=inputs.dtype, device=inputs.device)
+    kb = K // 2 if fmt_w == FMT_INT4 else K
+    ka = K // 2 if fmt_a == FMT_INT4 else K
+    gemm(codes, weights, [Range(0, K, scale_x, scale_w, 0, 0 if per_seg_x else 1, 0 if per_seg_w else 1)],
+         m=M, n=N, a_fmt=fmt_a, b_fmt=fmt_w, out_dtype=inputs.dtype, lda=ka, ldb=kb,
+         batch=S, batch_stride_a=M * ka, batch_stride_b=N * kb,
+         batch_stride_sx=1 if per_seg_x else M, batch_stride_sw=1 if per_seg_w else N, out=out)
+    return out
+
+
+def real_quantized_gemm_dual_scaled(fmt_a: str, fmt_w: str, inputs: torch.Tensor, weights: torch.Tensor,
+                                    pos_scale_x: torch.Tensor, neg_scale_x: torch.Tensor,
+                                    scale_w: torch.Tensor) -> torch.Tensor:
+    """``<prefix>_real_quantized_gemm_dual_scaled`` (segquant/src/real_quant/real_gemm.cu:752-894).
+
+    The activations are stored once, as the code of the branch each element
+    took; the GEMM reads them as two ranges (non-negative codes with the
+    positive scale, negative codes with the negative scale).
+    """
+    _check_contract(inputs, weights, fmt_w, pos_scale_x, neg_scale_x, scale_w)
+    S, M, N, K = _shapes(inputs, weights, fmt_w)
+    per_seg_x = pos_scale_x.numel() == S
+    per_seg_w = scale_w.numel() == S
+    if pos_scale_x.numel() != neg_scale_x.numel() or (not per_seg_x and pos_scale_x.numel() != S * M):
+        raise RuntimeError("pos/neg scale_x must both have S or S*M entries")
+    if not per_seg_w and scale_w.numel() != S * N:
+        raise RuntimeError(f"scale_w has {scale_w.numel()} entries, expected {S} or {S * N}")
+    codes = quantize(inputs.view(S * M, K), fmt_a, pos_scale_x, neg_scale_x, seg_rows=M,
+                     seg_stride=1 if per_seg_x else M, row_stride=0 if per_seg_x else 1, dual=True)
+    out = torch.empty((*inputs.shape[:-1], N), dtype=inputs.dtype, device=inputs.device)
+    kb = K // 2 if fmt_w == FMT_INT4 else K
+    rs, cs = (0 if per_seg_x else 1), (0 if per_seg_w else 1)
+    gemm(codes, weights,
+         [Range(0, K, pos_scale_x, scale_w, 2, rs, cs), Range(0, K, neg_scale_x, scale_w, 3, rs, cs)],
+         m=M, n=N, a_fmt=fmt_a, b_fmt=fmt_w, out_dtype=inputs.dtype, lda=K, ldb=kb,
+         batch=S, batch_stride_a=M * K, batch_stride_b=N * kb,
+         batch_stride_sx=1 if per_seg_x else M, batch_stride_sw=1 if per_seg_w else N, out=out)
+    return out
+
+
+def real_quantized_quantize_weights(fmt: str, weights: torch.Tensor, outputs: torch.Tensor, scale_w) -> None:
+    """``real_quantized_quantize_weights`` (segquant/src/real_quant/seg_utils.h:82-119):
+    a python float selects the one-scale overload, a tensor the per-row one."""
+    _need_cuda(weights, outputs)
+    if weights.dim() != 2 or not weights.is_contiguous() or not outputs.is_contiguous():
+        raise RuntimeError("tensor must be contiguous")
+    if outputs.dtype != code_dtype(fmt):
+        raise RuntimeError("tensor dtype failed")
+    n, k = weights.shape
+    need = n * k // 2 if fmt == FMT_INT4 else n * k
+    if fmt == FMT_INT4 and (n * k) % 2:
+        raise RuntimeError("Quantization to int4 requires the number of elements to be even")
+    if outputs.numel() != need:
+        raise RuntimeError("output numel must match the weight" + (" (half of it for int4)" if fmt == FMT_INT4 else ""))
+    lib = L.lib()
+    if isinstance(scale_w, torch.Tensor):
+        _need_cuda(scale_w)
+        if scale_w.dtype != torch.float32 or scale_w.numel() != n or not scale_w.is_contiguous():
+            raise RuntimeError("scale_w must be a contiguous float32 vector with one entry per row")
+        rc = lib.segq_quantize_weights_rows(weights.data_ptr(), _dt(weights.dtype), n, k, outputs.data_ptr(),
+                                            _CODE[fmt], scale_w.data_ptr(), _stream())
+    elif isinstance(scale_w, float):
+        rc = lib.segq_quantize_weights_scalar(weights.data_ptr(), _dt(weights.dtype), n, k, outputs.data_ptr(),
+                                              _CODE[fmt], C.c_float(scale_w), _stream())
+    else:  # the float overload is noconvert (seg_utils.h:99)
+        raise TypeError("scale_w must be a python float or a float32 tensor")
+    L.check(rc)
+
+
+def fake_e4m3fy(inputs: torch.Tensor) -> torch.Tensor:
+    """``fake_e4m3fy`` on the GPU (segquant/src/fake_quant/quantizer_fp8.cu:43-51)."""
+    _need_cuda(inputs)
+    x = inputs.contiguous()
+    out = torch.empty_like(x)
+    L.check(L.lib().segq_fake_e4m3(x.data_ptr(), out.data_ptr(), _dt(x.dtype), x.numel(), _stream()))
+    return out

@@ -1,0 +1,433 @@
+"""GPU parity tests of the HIP kernels against the CPU oracle, through the C ABI.
+
+Integer codes, int4 packing and int32 accumulators must be bit-exact.  The fp8
+MFMA sums each 128-long group of exact products with a limited-width aligned
+adder, so fp8 accumulators are compared with the exact fp64 sum to within
+FP8_ACC_TOL of sum |a||b| (measured: 4e-5 on codes drawn uniformly from the
+whole e4m3 range).  De-quantised outputs use the tolerances the path is
+specified with: 1e-3 relative for int8, 1e-2 for fp8 against the fp32
+fake-quant result.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import segq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+FP8_ACC_TOL = 2e-4
+FMTS = [O.FMT_INT8, O.FMT_E4M3, O.FMT_INT4]
+TDT = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from segquant_amd import ops as _ops
+    _ops.L.lib()  # fail loudly if the library is not built
+    return _ops
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy() if t.dtype in (torch.bfloat16, torch.float16) else t.detach().cpu().numpy()
+
+
+def _codes_np(t, fmt, cols=None):
+    a = t.cpu().numpy()
+    if fmt == O.FMT_INT4:
+        return np.stack([O.unpack_int4(r) for r in a.reshape(a.shape[0], -1)])
+    return a
+
+
+def _special_matrix(rows, cols, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g) * 3
+    x[0, :18] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 0.0, -0.0, 1e30, -1e30, float("inf"), float("-inf"),
+                              float("nan"), 126.5, 127.5, -127.5, -128.5, 1e-30])
+    return x.to(dtype)
+
+
+# ------------------------------------------------------------------ quantise
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("dt", ["fp32", "bf16", "fp16"])
+def test_quantize_per_tensor_and_per_row_bit_exact(ops, fmt, dt):
+    rows, cols = 37, 208
+    x = _special_matrix(rows, cols, 1, TDT[dt]).to(DEV)
+    xn = _np(x)
+    for per_row in (False, True):
+        s = (torch.rand(rows if per_row else 1) * 20 + 0.5).to(DEV)
+        c = ops.quantize(x, fmt, s, row_stride=1 if per_row else 0)
+        want = O.quantize_act(xn[None], s.cpu().numpy(), fmt)[0]
+        got = _codes_np(c, fmt)
+        assert np.array_equal(got, want), (fmt, dt, per_row)
+
+
+def test_e4m3_hardware_cast_on_every_midpoint(ops):
+    tab = O.e4m3_decode_table()
+    pos = np.sort(tab[:0x7F])
+    mids = ((pos[:-1].astype(np.float64) + pos[1:]) / 2).astype(np.float32)
+    pts = np.concatenate([pos, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+                          np.float32([449, 464, 465, 480, 1e9, np.inf])])
+    pts = np.concatenate([pts, -pts, np.float32([np.nan])])
+    pad = (-len(pts)) % 16
+    pts = np.concatenate([pts, np.zeros(pad, np.float32)])
+    x = torch.from_numpy(pts).view(1, -1).to(DEV)
+    one = torch.ones(1, device=DEV)
+    c = ops.quantize(x, O.FMT_E4M3, one).cpu().numpy()[0]
+    assert np.array_equal(c, O.e4m3_encode(pts))
+    rt = ops.fake_e4m3fy(x).cpu().numpy()[0]
+    want = O.e4m3_roundtrip(pts)
+    assert np.array_equal(np.isnan(rt), np.isnan(want))
+    assert np.array_equal(rt[~np.isnan(rt)], want[~np.isnan(want)])
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_quantize_reference_segment_indexing(ops, fmt):
+    S, B, M, K = 3, 2, 5, 64
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(S, B, M, K, generator=g) * 2).to(torch.bfloat16).to(DEV)
+    rows = B * M
+    for per_tok in (False, True):
+        s = (torch.rand(S * rows if per_tok else S, generator=g) * 30 + 1).to(DEV)
+        c = ops.quantize(x.view(S * rows, K), fmt, s, seg_rows=rows, seg_stride=rows if per_tok else 1,
+                         row_stride=1 if per_tok else 0)
+        want = O.quantize_act(_np(x), s.cpu().numpy(), fmt).reshape(S * rows, K)
+        assert np.array_equal(_codes_np(c, fmt), want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_quantize_dual_two_tensor_and_merged(ops, fmt):
+    S, M, K = 2, 9, 96
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(S, M, K, generator=g)
+    x[0, 0, :4] = torch.tensor([0.0, -0.0, float("nan"), -1e-20])
+    x = x.to(DEV)
+    pos = (torch.rand(S, generator=g) * 30 + 1).to(DEV)
+    neg = (torch.rand(S, generator=g) * 60 + 1).to(DEV)
+    xp, xn = ops.quantize(x.view(S * M, K), fmt, pos, neg, seg_rows=M, seg_stride=1, dual=True, two_tensors=True)
+    wp, wn = O.quantize_act_dual(_np(x), pos.cpu().numpy(), neg.cpu().numpy(), fmt)
+    assert np.array_equal(_codes_np(xp, fmt), wp.reshape(S * M, K))
+    assert np.array_equal(_codes_np(xn, fmt), wn.reshape(S * M, K))
+    merged = ops.quantize(x.view(S * M, K), fmt, pos, neg, seg_rows=M, seg_stride=1, dual=True)
+    want = O.merge_dual_codes(wp, wn, _np(x)).reshape(S * M, K)
+    assert np.array_equal(_codes_np(merged, fmt), want)
+
+
+def test_quantize_column_segments_with_partial_dual(ops):
+    M, K = 11, 160
+    bounds = [0, 48, 160]
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([10.0, 20.0], device=DEV)
+    neg = torch.tensor([99.0, 40.0], device=DEV)
+    c = ops.quantize(x, O.FMT_INT8, pos, neg, kseg_bounds=bounds, kseg_stride=1, dual=True, dual_kseg_mask=0b10)
+    xn = _np(x)
+    w0 = O.quantize_act(xn[None, :, :48], np.float32([10.0]), O.FMT_INT8)[0]
+    wp, wn = O.quantize_act_dual(xn[None, :, 48:], np.float32([20.0]), np.float32([40.0]), O.FMT_INT8)
+    w1 = O.merge_dual_codes(wp, wn, xn[None, :, 48:])[0]
+    assert np.array_equal(c.cpu().numpy(), np.concatenate([w0, w1], axis=1))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("dual", [False, True])
+def test_quantize_dynamic_per_row(ops, fmt, dual):
+    M, K = 13, 16 * 300  # longer than one cached pass of 256 threads
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g)
+    x[1] = x[1].abs()  # no negatives in this row
+    x[2] = 0
+    x = x.to(torch.bfloat16).to(DEV)
+    s = torch.empty(M, device=DEV)
+    sn = torch.empty(M, device=DEV) if dual else None
+    c = ops.quantize(x, fmt, s, sn, row_stride=1, dual=dual, dynamic=True)
+    xn = _np(x)
+    bits = 4 if fmt == O.FMT_INT4 else 8
+    if dual:
+        pa, na = O.dual_amax(xn, axis=-1)
+        ws, wn = O.fp8_dual_scales(pa, na) if fmt == O.FMT_E4M3 else O.int_dual_scales(pa, na, bits)
+        assert np.array_equal(s.cpu().numpy(), ws) and np.array_equal(sn.cpu().numpy(), wn)
+        wp, wq = O.quantize_act_dual(xn[None], ws, wn, fmt)
+        want = O.merge_dual_codes(wp, wq, xn[None])[0]
+    else:
+        amax = np.abs(xn).max(axis=-1)
+        ws = O.fp8_scale(amax) if fmt == O.FMT_E4M3 else O.int_scale(amax, bits)
+        assert np.array_equal(s.cpu().numpy(), ws)
+        want = O.quantize_act(xn[None], ws, fmt)[0]
+    assert np.array_equal(_codes_np(c, fmt), want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_quantize_weights_both_overloads(ops, fmt):
+    N, K = 24, 64
+    g = torch.Generator().manual_seed(6)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(DEV)
+    out = torch.empty(N * K // 2 if fmt == O.FMT_INT4 else (N, K), dtype=ops.code_dtype(fmt), device=DEV)
+    ops.real_quantized_quantize_weights(fmt, w, out, 311.5)
+    want = O.quantize_weights(_np(w), 311.5, fmt)
+    assert np.array_equal(_codes_np(out.view(N, -1), fmt), want)
+    s = (torch.rand(N, generator=g) * 300 + 50).to(DEV)
+    ops.real_quantized_quantize_weights(fmt, w, out, s)
+    want = O.quantize_weights(_np(w), s.cpu().numpy(), fmt)
+    assert np.array_equal(_codes_np(out.view(N, -1), fmt), want)
+    with pytest.raises(TypeError):
+        ops.real_quantized_quantize_weights(fmt, w, out, 3)
+
+
+# ------------------------------------------------------------------ GEMM accumulators
+def _rand_codes(shape, fmt, seed):
+    g = np.random.default_rng(seed)
+    if fmt == O.FMT_INT8:
+        c = g.integers(-128, 128, size=shape).astype(np.int8)
+        c.reshape(-1)[:7] = [-128, 127, -128, -128, 127, 0, -1]
+        return c
+    if fmt == O.FMT_INT4:
+        return g.integers(-8, 8, size=shape).astype(np.int8)
+    c = g.integers(0, 256, size=shape).astype(np.uint8)
+    c[(c & 0x7F) == 0x7F] = 0x3A  # no NaN codes
+    return c
+
+
+def _to_dev_codes(c, fmt):
+    if fmt == O.FMT_INT4:
+        return torch.from_numpy(np.stack([O.pack_int4(r) for r in c])).to(DEV)
+    return torch.from_numpy(c).to(DEV)
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("fa,fb", [(O.FMT_INT8, O.FMT_INT8), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_INT8, O.FMT_INT4)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (300, 200, 416), (3, 18, 64), (130, 515, 1056)])
+def test_gemm_raw_accumulators(ops, tile, fa, fb, M, N, K):
+    a = _rand_codes((M, K), fa, 10)
+    b = _rand_codes((N, K), fb, 11)
+    ad, bd = _to_dev_codes(a, fa), _to_dev_codes(b, fb)
+    ldb = K // 2 if fb == O.FMT_INT4 else K
+    out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], m=M, n=N, a_fmt=fa, b_fmt=fb, out_dtype="acc",
+                   lda=K, ldb=ldb, tile=tile)
+    ref = O.gemm_acc(a, b, fa, fb)
+    if fa == O.FMT_E4M3:
+        got = out.cpu().numpy().astype(np.float64)
+        mag = np.abs(O.code_values(a, fa)) @ np.abs(O.code_values(b, fb)).T
+        assert (np.abs(got - ref) <= FP8_ACC_TOL * mag + 1e-30).all()
+    else:
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+def test_gemm_sign_selected_halves_of_merged_codes(ops, fmt):
+    M, N, K = 70, 90, 320
+    a = _rand_codes((M, K), fmt, 12)
+    b = _rand_codes((N, K), fmt, 13)
+    ad, bd = _to_dev_codes(a, fmt), _to_dev_codes(b, fmt)
+    av = O.code_values(a, fmt)
+    neg = (a.view(np.uint8) & 0x80) != 0 if fmt == O.FMT_E4M3 else a < 0
+    for sel, keep in ((2, ~neg), (3, neg)):
+        out = ops.gemm(ad, bd, [ops.Range(0, K, None, None, a_sel=sel)], m=M, n=N, a_fmt=fmt, b_fmt=fmt,
+                       out_dtype="acc", lda=K, ldb=K)
+        ref = np.where(keep, av, 0.0) @ O.code_values(b, fmt).T
+        got = out.cpu().numpy().astype(np.float64)
+        if fmt == O.FMT_INT8:
+            assert np.array_equal(got, ref)
+        else:
+            assert (np.abs(got - ref) <= FP8_ACC_TOL * (np.abs(av) @ np.abs(O.code_values(b, fmt)).T) + 1e-30).all()
+
+
+def test_gemm_batched_sub_range_and_second_tensor(ops):
+    S, M, N, K = 3, 40, 50, 256
+    a = _rand_codes((S, M, K), O.FMT_INT8, 14)
+    a2 = _rand_codes((S, M, K), O.FMT_INT8, 15)
+    b = _rand_codes((S, N, K), O.FMT_INT8, 16)
+    ad, a2d, bd = (torch.from_numpy(t).to(DEV) for t in (a, a2, b))
+    out = ops.gemm(ad, bd, [ops.Range(64, 96, None, None, a_sel=1)], m=M, n=N, a_fmt=O.FMT_INT8,
+                   b_fmt=O.FMT_INT8, out_dtype="acc", lda=K, ldb=K, a_neg=a2d, batch=S,
+                   batch_stride_a=M * K, batch_stride_b=N * K)
+    for s in range(S):
+        ref = O.gemm_acc(a2[s][:, 64:160], b[s][:, 64:160], O.FMT_INT8, O.FMT_INT8)
+        assert np.array_equal(out[s].cpu().numpy().astype(np.int64), ref.astype(np.int64))
+
+
+# ------------------------------------------------------------------ fused epilogue
+@pytest.mark.parametrize("odt", ["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("fa,fb", [(O.FMT_INT8, O.FMT_INT8), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_INT8, O.FMT_INT4)])
+def test_gemm_dequant_bias_all_scale_shapes(ops, odt, fa, fb):
+    M, N, K = 77, 133, 192
+    a = _rand_codes((M, K), fa, 20)
+    b = _rand_codes((N, K), fb, 21)
+    if fa == O.FMT_E4M3:  # keep magnitudes finite in fp16
+        a &= 0xBF
+        b &= 0xBF
+    ad, bd = _to_dev_codes(a, fa), _to_dev_codes(b, fb)
+    g = torch.Generator().manual_seed(22)
+    bias = torch.randn(N, generator=g).to(DEV)
+    acc = O.gemm_acc(a, b, fa, fb)
+    mag = np.abs(O.code_values(a, fa)) @ np.abs(O.code_values(b, fb)).T
+    for per_row in (False, True):
+        for per_col in (False, True):
+            sx = (torch.rand(M if per_row else 1, generator=g) * 50 + 1).to(DEV)
+            sw = (torch.rand(N if per_col else 1, generator=g) * 500 + 1).to(DEV)
+            out = ops.gemm(ad, bd, [ops.Range(0, K, sx, sw, 0, int(per_row), int(per_col))], m=M, n=N,
+                           a_fmt=fa, b_fmt=fb, out_dtype=TDT[odt], lda=K, ldb=K // 2 if fb == O.FMT_INT4 else K,
+                           bias=bias)
+            sxn = np.broadcast_to(sx.cpu().numpy().reshape(-1, 1), (M, 1))
+            swn = np.broadcast_to(sw.cpu().numpy().reshape(1, -1), (1, N))
+            exact = acc / (sxn.astype(np.float64) * swn) + bias.cpu().numpy()
+            got = _np(out).astype(np.float64)
+            if fa == O.FMT_E4M3:
+                ulp = {"fp32": 0.0, "bf16": 2.0 ** -8, "fp16": 2.0 ** -11}[odt]
+                tol = FP8_ACC_TOL * mag / (sxn.astype(np.float64) * swn) + ulp * np.abs(exact) + 1e-6
+                assert (np.abs(got - exact) <= tol).all()
+            elif odt == "fp32":
+                assert np.abs(got - exact).max() <= 2e-6 * np.abs(exact).max()
+            else:
+                want = O.round_to_dtype(exact.astype(np.float32), odt).astype(np.float64)
+                ulp = 2.0 ** (-7 if odt == "bf16" else -10)
+                assert (np.abs(got - want) <= ulp * np.abs(want) + 1e-30).all()
+                assert (got != want).mean() < 1e-3  # only ties flip
+
+
+def test_gemm_fold_two_k_segments_plus_dual(ops):
+    """K = [attn | mlp]: segment 0 single scale, segment 1 DualScale -> three ranges."""
+    M, N, K0, K1 = 150, 200, 128, 320
+    K = K0 + K1
+    g = torch.Generator().manual_seed(30)
+    x = torch.randn(M, K, generator=g)
+    x[:, K0:] = torch.nn.functional.gelu(x[:, K0:] * 2, approximate="tanh")
+    w = torch.randn(N, K, generator=g) * 0.02
+    xn, wn = x.numpy(), w.numpy()
+    s0 = np.float32(O.int_scale(float(np.abs(xn[:, :K0]).max())))
+    pa, na = O.dual_amax(xn[:, K0:])
+    ps, ns = (np.float32(t) for t in O.int_dual_scales(pa, na))
+    sw = np.float32(O.int_scale(float(np.abs(wn).max())))
+    wq = O.quantize_weights(wn, float(sw), O.FMT_INT8)
+    xd = x.to(DEV)
+    pos = torch.tensor([s0, ps], device=DEV)
+    neg = torch.tensor([s0, ns], device=DEV)
+    swd = torch.tensor([sw], device=DEV)
+    codes = ops.quantize(xd, O.FMT_INT8, pos, neg, kseg_bounds=[0, K0, K], kseg_stride=1, dual=True,
+                         dual_kseg_mask=0b10)
+    bias = torch.randn(N, generator=g).to(DEV)
+    ranges = [ops.Range(0, K0, pos[0:1], swd, 0), ops.Range(K0, K1, pos[1:2], swd, 2),
+              ops.Range(K0, K1, neg[1:2], swd, 3)]
+    for tile in (2, 3, 4, 5):
+        out = ops.gemm(codes, torch.from_numpy(wq).to(DEV), ranges, m=M, n=N, a_fmt=O.FMT_INT8,
+                       b_fmt=O.FMT_INT8, out_dtype=torch.float32, lda=K, ldb=K, bias=bias, tile=tile)
+        # oracle: three exact partial sums, each divided by its scales
+        c0 = O.quantize_act(xn[None, :, :K0], [s0], O.FMT_INT8)[0]
+        cp, cn = O.quantize_act_dual(xn[None, :, K0:], [ps], [ns], O.FMT_INT8)
+        y = (O.gemm_acc(c0, wq[:, :K0], O.FMT_INT8, O.FMT_INT8) / (np.float64(s0) * sw)
+             + O.gemm_acc(cp[0], wq[:, K0:], O.FMT_INT8, O.FMT_INT8) / (np.float64(ps) * sw)
+             + O.gemm_acc(cn[0], wq[:, K0:], O.FMT_INT8, O.FMT_INT8) / (np.float64(ns) * sw)
+             + bias.cpu().numpy())
+        got = out.cpu().numpy().astype(np.float64)
+        assert np.abs(got - y).max() <= 1e-5 * np.abs(y).max(), tile
+        # and within the path's tolerance of the fp32 fake-quant linear
+        xf = np.concatenate([O.fake_quant_int(xn[:, :K0], s0), O.fake_quant_int_dual(xn[:, K0:], ps, ns)], axis=1)
+        ref = xf @ O.fake_quant_int(wn, sw).T + bias.cpu().numpy()
+        assert np.abs(got - ref).max() <= 1e-3 * np.abs(ref).max()
+
+
+# ------------------------------------------------------------------ the reference's op contract
+GRID = [(O.FMT_INT8, O.FMT_INT8, 1e-3), (O.FMT_E4M3, O.FMT_E4M3, 1e-2), (O.FMT_INT8, O.FMT_INT4, 1e-3)]
+
+
+def _fake(x, fmt, s):
+    return O.fake_quant_fp8(x, s) if fmt == O.FMT_E4M3 else O.fake_quant_int(x, s, 4 if fmt == O.FMT_INT4 else 8)
+
+
+def _scale_of(amax, fmt):
+    return O.fp8_scale(amax) if fmt == O.FMT_E4M3 else O.int_scale(amax, 4 if fmt == O.FMT_INT4 else 8)
+
+
+@pytest.mark.parametrize("fa,fw,tol", GRID)
+@pytest.mark.parametrize("axis", [False, True])
+@pytest.mark.parametrize("seg", ["none", "weight", "input"])
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_reference_contract_scaled(ops, fa, fw, tol, axis, seg, dt):
+    """Same grid as the reference's test_mix_real (test/test_linear.py:901-913):
+    types x per-tensor / per-token+per-channel x segmentation."""
+    B, Mtok, K, N = 2, 3, 256, 192
+    S = 1 if seg == "none" else 2
+    g = torch.Generator().manual_seed(40)
+    x = torch.randn(B, Mtok, K, generator=g).to(TDT[dt])
+    w = torch.randn(N, K, generator=g) * 0.02
+    xs, ws = O.segment_views(_np(x), w.numpy(), "weight" if seg == "none" else seg, S)
+    xs = np.ascontiguousarray(xs)
+    ws = np.ascontiguousarray(ws)
+    M = B * Mtok
+    if axis:
+        sx = np.stack([_scale_of(np.abs(xs[s]).reshape(M, -1).max(-1), fa) for s in range(S)]).astype(np.float32)
+        sw = np.stack([_scale_of(np.abs(ws[s]).max(-1), fw) for s in range(S)]).astype(np.float32)
+    else:
+        sx = np.float32([_scale_of(float(np.abs(xs[s]).max()), fa) for s in range(S)])
+        sw = np.float32([_scale_of(float(np.abs(ws[s]).max()), fw) for s in range(S)])
+    wq = np.stack([O.quantize_weights(ws[s], sw[s] if axis else float(sw[s]), fw) for s in range(S)])
+    wq_dev = (torch.from_numpy(np.stack([O.pack_int4(wq[s]) for s in range(S)])) if fw == O.FMT_INT4
+              else torch.from_numpy(wq)).to(DEV)
+    xin = torch.from_numpy(xs).to(TDT[dt]).to(DEV)
+    out = ops.real_quantized_gemm_scaled(fa, fw, xin, wq_dev, torch.from_numpy(sx).to(DEV),
+                                         torch.from_numpy(sw).to(DEV))
+    assert out.shape == (S, B, Mtok, ws.shape[1]) and out.dtype == TDT[dt]
+    # oracle of the real pipeline (same codes): tight
+    wq_or = wq_dev.cpu().numpy()
+    want = O.real_quantized_gemm_scaled(xs, wq_or, sx, sw, fa, fw, out_dtype=dt)
+    got = _np(out).astype(np.float64)
+    ulp = {"fp32": 2e-6, "bf16": 2.0 ** -7}[dt]
+    if fa == O.FMT_E4M3:
+        ulp += 1e-3  # limited-width accumulation inside the fp8 MFMA
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= ulp * scale
+    # fp32 fake-quant reference: the path's stated tolerance (fp32 output only;
+    # a bf16 result carries its own 2^-9 rounding)
+    if dt == "fp32":
+        sxb = sx.reshape(S, M, 1) if axis else sx.reshape(S, 1, 1)
+        swb = sw.reshape(S, -1, 1) if axis else sw.reshape(S, 1, 1)
+        xf = np.stack([_fake(xs[s].reshape(M, -1), fa, sxb[s]) for s in range(S)])
+        wf = np.stack([_fake(ws[s], fw, swb[s]) for s in range(S)])
+        ref = O.segmented_matmul(xf, wf).reshape(got.shape)
+        assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("fa,fw,tol", GRID)
+@pytest.mark.parametrize("axis", [False, True])
+def test_reference_contract_dual_scaled(ops, fa, fw, tol, axis):
+    S, M, K, N = 2, 10, 128, 96
+    g = torch.Generator().manual_seed(41)
+    x = torch.nn.functional.silu(torch.randn(S, M, K, generator=g) * 3)
+    w = torch.randn(S, N, K, generator=g) * 0.02
+    xn, wn = x.numpy(), w.numpy()
+    bits_a = 8
+    if axis:
+        pa, na = O.dual_amax(xn, axis=-1)
+        ps, ns = O.fp8_dual_scales(pa, na) if fa == O.FMT_E4M3 else O.int_dual_scales(pa, na, bits_a)
+        sw = np.stack([_scale_of(np.abs(wn[s]).max(-1), fw) for s in range(S)]).astype(np.float32)
+    else:
+        pn = [O.dual_amax(xn[s]) for s in range(S)]
+        sc = [O.fp8_dual_scales(*t) if fa == O.FMT_E4M3 else O.int_dual_scales(*t, bits_a) for t in pn]
+        ps, ns = np.float32([t[0] for t in sc]), np.float32([t[1] for t in sc])
+        sw = np.float32([_scale_of(float(np.abs(wn[s]).max()), fw) for s in range(S)])
+    wq = np.stack([O.quantize_weights(wn[s], sw[s] if axis else float(sw[s]), fw) for s in range(S)])
+    wq_dev = (torch.from_numpy(np.stack([O.pack_int4(wq[s]) for s in range(S)])) if fw == O.FMT_INT4
+              else torch.from_numpy(wq)).to(DEV)
+    out = ops.real_quantized_gemm_dual_scaled(fa, fw, x.to(DEV), wq_dev, torch.from_numpy(np.float32(ps)).to(DEV),
+                                              torch.from_numpy(np.float32(ns)).to(DEV), torch.from_numpy(sw).to(DEV))
+    want = O.real_quantized_gemm_dual_scaled(xn, wq_dev.cpu().numpy(), ps, ns, sw, fa, fw)
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= (1e-3 if fa == O.FMT_E4M3 else 3e-6) * np.abs(want).max()
+    psb = np.float32(ps).reshape(S, -1, 1)
+    nsb = np.float32(ns).reshape(S, -1, 1)
+    swb = sw.reshape(S, -1, 1)
+    xf = np.stack([(O.fake_quant_fp8_dual(xn[s], psb[s], nsb[s]) if fa == O.FMT_E4M3
+                    else O.fake_quant_int_dual(xn[s], psb[s], nsb[s])) for s in range(S)])
+    wf = np.stack([_fake(wn[s], fw, swb[s]) for s in range(S)])
+    ref = O.segmented_matmul(xf, wf)
+    assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
+
+
+def test_errors_are_runtime_errors(ops):
+    x = torch.randn(1, 4, 40, device=DEV)  # K = 40 is not a multiple of 16
+    w = torch.zeros(1, 8, 40, dtype=torch.int8, device=DEV)
+    s = torch.ones(1, device=DEV)
+    with pytest.raises(RuntimeError):
+        ops.real_quantized_gemm_scaled(O.FMT_INT8, O.FMT_INT8, x, w, s, s)
+    with pytest.raises(RuntimeError):
+        ops.real_quantized_gemm_scaled(O.FMT_INT8, O.FMT_INT8, x.cpu(), w, s, s)
