@@ -1,0 +1,158 @@
+#!/usr/bin/env python3
+"""Benchmark of the real-quantised segmented linear on one MI355X.
+
+A step is one pass of the hot path (activation quantise -> segmented MFMA GEMM
+with fused de-quantisation and bias) over every linear of the workload, on
+synthetic inputs already resident in HBM.  The default workload is the FLUX.1
+double-stream block at M = 4608, INT8 W8A8 (the configuration the headline
+metric is quoted on).  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TOPS = {"int8": 5000.0, "fpe4m3": 5000.0}  # dense MFMA, TOP/s
+PEAK_HBM = 8000.0                               # GB/s
+
+
+def cpu_baseline(specs, rows, repeats=3):
+    """The fake-quant path (fp32 quantise->de-quantise + torch matmul) on the
+    host cores, on the first ``rows`` tokens of every linear of the workload."""
+    import torch
+    from oracle import fake_path_torch as F
+    from segquant_amd import workloads as W
+    cores = os.cpu_count() or 1
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(threads)
+    work = []
+    ops = 0
+    for sp in specs:
+        x = W.make_input(sp, M=rows)
+        w = W.make_weight(sp)
+        # weights are fake-quantised once, offline, and stored de-quantised
+        if sp.weight_axis == 1:
+            ws = F.scale_of(w.abs().amax(dim=1, keepdim=True), sp.weight)
+            w_hat = F.fake_quant(w, sp.weight, ws)
+        elif sp.seg_mode == "weight" and sp.chunksizes:
+            w_hat = torch.cat([F.fake_quant(b, sp.weight, F.scale_of(b.abs().amax(), sp.weight))
+                               for b in w.split(sp.chunksizes, dim=0)])
+        else:
+            w_hat = F.fake_quant(w, sp.weight, F.scale_of(w.abs().amax(), sp.weight))
+        bounds = W.segment_bounds(sp)
+        n_in = len(bounds) - 1
+        dual = [i in sp.dual_segments for i in range(n_in)]
+        work.append((x, w_hat, W.make_bias(sp), sp.act, bounds, dual, sp.act_axis == -1))
+        ops += 2 * rows * sp.N * sp.K
+    times = []
+    for it in range(repeats + 1):
+        t0 = time.perf_counter()
+        for args in work:
+            F.fake_linear(*args)
+        t1 = time.perf_counter()
+        if it:  # first pass is the warm-up
+            times.append(t1 - t0)
+    t = sorted(times)[len(times) // 2]
+    return {"value": ops / t / 1e12, "unit": "TOP/s", "cores": threads, "kind": "port",
+            "sample": f"first {rows} of {specs[0].M} tokens of each linear, fp32 fake-quant + torch.matmul, "
+                      f"median of {repeats} passes, {t:.3f} s per pass"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=3, help="benchmark configuration 1..5 (default: FLUX int8, M=4608)")
+    ap.add_argument("--cpu-rows", type=int, default=512, help="tokens per linear in the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from segquant_amd import ops, workloads as W
+    from segquant_amd._lib import lib
+    lib()  # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    specs = W.config_linears(args.config)
+    layers, inputs = [], []
+    bytes_per_set = 0
+    for sp in specs:
+        layer, x = W.build_layer(sp, device=dev, real_quant=True)
+        assert layer.optimizer.real_quant
+        layers.append(layer)
+        inputs.append(x.to(sp.x_dtype))
+        bytes_per_set += sp.M * sp.K * (x.to(sp.x_dtype).element_size() + 1) + sp.M * sp.N * 2
+    # rotate over enough input copies that a step never finds its operands in the
+    # 256 MB last-level cache left there by the previous step
+    n_sets = max(2, -(-(768 << 20) // bytes_per_set))
+    sets = [[x.to(dev).clone() for x in inputs] for _ in range(n_sets)]
+
+    def step(i):
+        xs = sets[i % n_sets]
+        for layer, x in zip(layers, xs):
+            layer(x)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    with ops.record_launches() as log:
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(args.warmup + i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    wall = t1 - t0
+    total_ops = sum(sp.ops for sp in specs)
+    value = total_ops * args.steps / wall / 1e12
+
+    g_t = g_ops = g_exec = q_t = q_bytes = 0.0
+    n_g = n_q = 0
+    for kind, e0, e1, info in log:
+        ms = e0.elapsed_time(e1)
+        if kind == "gemm":
+            g_t += ms * 1e-3
+            g_ops += 2.0 * info["m"] * info["n"] * info["k_alg"] * info["batch"]
+            g_exec += 2.0 * info["m"] * info["n"] * info["k_exec"] * info["batch"]
+            n_g += 1
+        else:
+            q_t += ms * 1e-3
+            q_bytes += info["rows"] * info["cols"] * (info["x_bytes"] + info["code_bytes"] * info["tensors"])
+            n_q += 1
+    fmt = specs[0].act
+    peak = PEAK_TOPS[fmt]
+    g_tops = g_ops / g_t / 1e12
+    q_gbs = q_bytes / q_t / 1e9
+    out = {
+        "metric": "seg-GEMM TOPS + % MFMA peak (FLUX shapes, M=4608); quantize kernel GB/s",
+        "value": round(value, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8" if fmt == "int8" else "fp8_e4m3", "data": "synthetic",
+        "config": {"workload": f"config {args.config}: " + ", ".join(f"{s.name} M{s.M} K{s.K} N{s.N} {s.kernel_type}" for s in specs),
+                   "step": "activation quantize + segmented GEMM with fused dequant+bias, per linear",
+                   "input_dtype": str(specs[0].x_dtype).replace("torch.", ""), "output_dtype": str(specs[0].x_dtype).replace("torch.", "")},
+        "roofline": {"bound": "mfma", "kernel": "segq::gemm_kernel", "achieved": round(g_tops, 2), "peak": peak,
+                     "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": None,
+                     "launches": n_g, "avg_launch_us": round(g_t / max(n_g, 1) * 1e6, 2),
+                     "executed_tops": round(g_exec / g_t / 1e12, 2)},
+        "quantize": {"bound": "hbm", "kernel": "segq::quant_*_kernel", "achieved": round(q_gbs, 1), "peak": PEAK_HBM,
+                     "unit": "GB/s", "frac": round(q_gbs / PEAK_HBM, 4), "launches": n_q,
+                     "avg_launch_us": round(q_t / max(n_q, 1) * 1e6, 2)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(specs, args.cpu_rows)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

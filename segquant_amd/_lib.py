@@ -82,6 +82,10 @@ def lib() -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    # torch ships its own HIP runtime; it has to be in the process before this
+    # library is, so that both resolve to the same runtime (two runtimes in one
+    # process do not see each other's devices and streams)
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with `make -C {CSRC_DIR}` "

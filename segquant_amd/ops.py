@@ -49,6 +49,43 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+# When set to a list, every quantise / GEMM launch is bracketed by events on the
+# launching stream and (kind, start, end, info) is appended; see record_launches.
+_launch_log = None
+
+
+class record_launches:
+    """Context manager: collect (kind, start_event, end_event, info) for each
+    kernel launch made through this module.  Read ``elapsed_time`` after a
+    device synchronisation."""
+
+    def __init__(self):
+        self.log = []
+
+    def __enter__(self):
+        global _launch_log
+        self._prev = _launch_log
+        _launch_log = self.log
+        return self.log
+
+    def __exit__(self, *exc):
+        global _launch_log
+        _launch_log = self._prev
+        return False
+
+
+def _launch(kind, info, fn):
+    if _launch_log is None:
+        return fn()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    rc = fn()
+    e1.record()
+    _launch_log.append((kind, e0, e1, info))
+    return rc
+
+
 def code_dtype(fmt: str) -> torch.dtype:
     """Storage dtype of codes: int8 as int8, e4m3 and packed int4 as uint8
     (segquant/src/real_quant/seg_utils.h:25-45)."""
@@ -98,7 +135,9 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
         for i, b in enumerate(kseg_bounds):
             d.kseg_bounds[i] = int(b)
     d.dual = 1 if dual else 0; d.dual_kseg_mask = dual_kseg_mask & 0xFFFFFFFF; d.dynamic = 1 if dynamic else 0
-    L.check(L.lib().segq_quantize(C.byref(d), _stream()))
+    info = dict(rows=rows, cols=cols, x_bytes=x.element_size(), code_bytes=0.5 if fmt == FMT_INT4 else 1.0,
+                tensors=2 if two_tensors else 1, dynamic=bool(dynamic))
+    L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
     return (out, out_neg) if two_tensors else out
 
 
@@ -161,7 +200,9 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
                 raise RuntimeError("scales must be float32")
         kr.sx = r.sx.data_ptr() if r.sx is not None else None
         kr.sw = r.sw.data_ptr() if r.sw is not None else None
-    L.check(L.lib().segq_gemm(C.byref(d), _stream()))
+    info = dict(m=m, n=n, batch=batch, k_alg=sum(r.k_len for r in ranges if r.a_sel in (0, 2)),
+                k_exec=sum(r.k_len for r in ranges), a_fmt=a_fmt, b_fmt=b_fmt)
+    L.check(_launch("gemm", info, lambda: L.lib().segq_gemm(C.byref(d), _stream())))
     return out
 
 

@@ -1,0 +1,288 @@
+"""The optimiser owns the quantised weights and scales of one segmented linear
+and is the single call site of the kernels.
+
+Counterpart of ``BaseOptimizer`` / ``DefaultOptimizer``
+(segquant/optimum/optimizer.py:10-123, :147-293).  Two routes reach the GPU:
+
+* :meth:`BaseOptimizer.call_func` keeps the reference's call
+  ``ext_dict[kernel_type][func_name](X, W, scales...)`` on ``(S, ...)`` tensors
+  and returns per-segment outputs.
+* :meth:`DefaultOptimizer.forward_fused` is this build's own route: one
+  quantise launch and one GEMM launch on the un-replicated input, segments
+  expressed as a per-column scale vector (weight-seg) or K ranges (input-seg),
+  bias added in the epilogue, output already in its final layout.
+
+The smoothing and low-rank optimisers of the reference are calibration-time
+algebra outside the kernel path and are not built.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from ..layers import ext_dict
+from ..layers.segment_tensor_manager import InputSegmentTensorManager, segmented_matmul
+
+_FMT = {"int8": ops.FMT_INT8, "int4": ops.FMT_INT4, "fpe4m3": ops.FMT_E4M3}
+
+
+def _as_f32(v, device):
+    if isinstance(v, torch.Tensor):
+        return v.to(dtype=torch.float32, device=device)
+    return torch.tensor(v, dtype=torch.float32, device=device)
+
+
+class BaseOptimizer:
+    def __init__(self, seg_mode, chunks, chunksizes, weight_manager, input_calibrators, weight_calibrators,
+                 real_quant=False, dual_scale=False, kernel_type=None, dual_segments=None):
+        self.seg_mode = seg_mode
+        self.chunks = chunks
+        self.chunksizes = chunksizes
+        self.weight_manager = weight_manager
+        self.input_calibrators = input_calibrators
+        self.weight_calibrators = weight_calibrators
+        self.real_quant = real_quant
+        self.kernel_type = kernel_type
+        self.packed = bool(real_quant and "Wint4" in (kernel_type or ""))
+        self.dual_scale = dual_scale
+        # which input calibrators are DualScale (this build allows a mix: e.g. the
+        # attention half of a concatenated input single-scale, the MLP half dual)
+        self.dual_segments = list(dual_segments) if dual_segments is not None else [dual_scale] * len(input_calibrators)
+        self.func_name = "gemm_dual_scaled_fn" if (real_quant and dual_scale) else "gemm_scaled_fn"
+        self.has_calibrated = False
+        self.scale_tensor = None
+        self._plan = None
+
+    def _stack(self, calibrators, attr):
+        dev = self.weight_manager.device()
+
+        def pick(c):
+            v = getattr(c, attr)
+            # a single-scale quantiser in a DualScale layer uses its one scale for both signs
+            return c.scale if v is None and attr in ("pos_scale", "neg_scale") else v
+
+        vals = [_as_f32(pick(c), dev) for c in calibrators]
+        if len(vals) == 1:
+            vals = vals * self.chunks
+        if len({tuple(v.shape) for v in vals}) != 1:
+            return None  # unequal segments: only the fused route and the fake path apply
+        return torch.stack(vals)
+
+    def make_scale_tensor(self):
+        """(S,) or (S, M) input scales and (S,) or (S, n) weight scales, fp32 on
+        the weight's device; DualScale gives (pos, neg, weight)."""
+        w = self._stack(self.weight_calibrators, "scale")
+        if self.dual_scale:
+            self.scale_tensor = (self._stack(self.input_calibrators, "pos_scale"),
+                                 self._stack(self.input_calibrators, "neg_scale"), w)
+        else:
+            self.scale_tensor = (self._stack(self.input_calibrators, "scale"), w)
+        self._plan = None
+
+    def call_func(self, batch_input: torch.Tensor, batch_weight: torch.Tensor):
+        if self.real_quant:
+            if self.input_calibrators[0].dynamic:
+                # The reference calls a method that does not exist here
+                # (optimizer.py:96-100).  Recalibrate each segment on this
+                # input instead; the fused route does this inside the kernel.
+                for cal, chunk in zip(self.input_calibrators, batch_input):
+                    cal.reset()
+                    cal.calibrate(chunk)
+                self.make_scale_tensor()
+            fn = ext_dict[self.kernel_type][self.func_name]
+            args = [t.contiguous() for t in self.scale_tensor]
+            return fn(batch_input.contiguous(), batch_weight.contiguous(), *args)
+        # fake path: quantise-dequantise each segment, then a float matmul.
+        # The input is not modified (the reference writes into a view of it).
+        quantised = torch.stack([self.input_calibrators[min(i, len(self.input_calibrators) - 1)].quantize(seg)
+                                 for i, seg in enumerate(batch_input)])
+        return segmented_matmul(quantised, batch_weight)
+
+    def process_step(self, err):
+        pass
+
+    def to_cpu(self):
+        self._move("cpu")
+
+    def to_cuda(self, device):
+        self._move(device)
+
+    def _move(self, device):
+        self.weight_manager = self.weight_manager.to(device)
+        self.input_calibrators = [c.to(device) for c in self.input_calibrators]
+        self.weight_calibrators = [c.to(device) for c in self.weight_calibrators]
+        if self.scale_tensor is not None:
+            self.scale_tensor = tuple(t.to(device) if t is not None else None for t in self.scale_tensor)
+        self._plan = None
+
+
+class OptimizerRegistry:
+    _registry = {}
+
+    @classmethod
+    def register(cls, name):
+        def wrap(c):
+            cls._registry[name] = c
+            return c
+        return wrap
+
+    @classmethod
+    def get(cls, name):
+        return cls._registry.get(name)
+
+    @classmethod
+    def create(cls, name, **kwargs):
+        c = cls.get(name)
+        if c is None:
+            raise ValueError(f"Optimizer '{name}' not found in registry.")
+        return c(**kwargs)
+
+
+@OptimizerRegistry.register("default")
+class DefaultOptimizer(BaseOptimizer):
+    def __init__(self, seg_mode, chunks, chunksizes, weight_manager, input_calibrators, weight_calibrators,
+                 real_quant=False, dual_scale=False, kernel_type=None, dual_segments=None, **kwargs):
+        assert len(input_calibrators) == 1 or len(weight_calibrators) == 1, \
+            "Either input_calibrators or weight_calibrators must have a length of 1."
+        if seg_mode not in ("input", "weight"):
+            raise ValueError("seg_mode not found")
+        super().__init__(seg_mode, chunks, chunksizes, weight_manager, input_calibrators, weight_calibrators,
+                         real_quant, dual_scale, kernel_type, dual_segments)
+
+    def __repr__(self):
+        head = f"DefaultOptimizer(type={self.kernel_type}\n" if self.real_quant else "DefaultOptimizer(\n"
+        iq = ",\n    ".join(repr(c) for c in self.input_calibrators)
+        wq = ",\n    ".join(repr(c) for c in self.weight_calibrators)
+        return head + f"    input_quantizers=[\n    {iq}\n  ],\n    weight_quantizers=[\n    {wq}\n  ]\n)"
+
+    def _input_segments(self, x):
+        """The tensor each input calibrator sees: column blocks for input
+        segmentation (sizes may differ), the whole input otherwise."""
+        if self.seg_mode == "input":
+            return x.split(self.chunksizes, dim=-1)
+        return [x]
+
+    def calibrate(self, input_manager: InputSegmentTensorManager):
+        x = input_manager.input_tensor
+        for cal, chunk in zip(self.input_calibrators, self._input_segments(x)):
+            cal.calibrate(chunk)
+        w = self.weight_manager.weight_tensor
+        # input-seg: one weight calibrator sees the whole matrix; weight-seg: one per row block
+        blocks = [w] if self.seg_mode == "input" else w.split(self.chunksizes, dim=0)
+        for cal, wb in zip(self.weight_calibrators, blocks):
+            cal.calibrate(wb, input_data=x)
+
+    def finish_calibrate(self):
+        for i, cal in enumerate(self.input_calibrators):
+            cal.finish_calibrate()
+            self.input_calibrators[i] = cal.quantizer
+        wm = self.weight_manager
+        w = wm.weight_tensor
+        blocks = [w] if self.seg_mode == "input" else w.split(self.chunksizes, dim=0)
+        parts = []
+        for i, (cal, wb) in enumerate(zip(self.weight_calibrators, blocks)):
+            parts.append(cal.finish_calibrate(wb.contiguous()).reshape(wb.shape[0], -1))
+            self.weight_calibrators[i] = cal.quantizer
+        # codes (or fake-quantised floats) stay in the (out, in) layout; packed
+        # int4 is (out, in/2) bytes, so K segments are byte ranges of each row
+        wm.weight_tensor = torch.cat(parts, dim=0) if len(parts) > 1 else parts[0]
+        wm.packed = self.packed
+        self.has_calibrated = True
+        self.make_scale_tensor()
+
+    def forward(self, input_manager: InputSegmentTensorManager):
+        """Per-segment outputs (S, ..., n) through the reference-convention
+        operator; needs equal segment sizes, as the reference does."""
+        if len(set(self.chunksizes)) != 1:
+            raise NotImplementedError("Only support equal chunksizes.")
+        return self.call_func(input_manager.iter_view(), self.weight_manager.iter_view())
+
+    def forward_fake(self, x: torch.Tensor) -> torch.Tensor:
+        """Fake-quantised linear without bias for any segment sizes: quantise-
+        dequantise each input block with its own scale, one float matmul."""
+        cals = self.input_calibrators
+        xq = torch.cat([c.quantize(seg) for c, seg in zip(cals, self._input_segments(x))], dim=-1)
+        return xq @ self.weight_manager.weight_tensor.to(xq.dtype).transpose(-1, -2)
+
+    # ---- the fused route -------------------------------------------------
+    def fused_available(self) -> bool:
+        return self.real_quant and self.has_calibrated
+
+    def _build_plan(self, device):
+        """Turns segments and calibrated scales into what the kernels take."""
+        wm = self.weight_manager
+        N, K = wm.out_features, wm.in_features
+        S = self.chunks
+        fa = _FMT[self.kernel_type.split("A", 1)[1]]
+        fw = _FMT[self.kernel_type[1:].split("A", 1)[0]]
+        wcodes = wm.weight_tensor
+        wcodes = wcodes.reshape(N, K // 2 if fw == ops.FMT_INT4 else K).contiguous()
+        dev = wm.device()
+        wscales = [_as_f32(c.scale, dev).reshape(-1) for c in self.weight_calibrators]
+        if self.seg_mode == "weight":
+            # per-segment or per-channel -> one scale per output column (or a single scalar)
+            if S == 1:
+                sw_vec = wscales[0]
+            else:
+                sw_vec = torch.cat([w.expand(n) if w.numel() == 1 else w for w, n in zip(wscales, self.chunksizes)])
+            bounds = [0, K]
+        else:
+            sw_vec = wscales[0]  # one calibrator for the whole matrix
+            bounds = [0]
+            for c in self.chunksizes:
+                bounds.append(bounds[-1] + c)
+        self._plan = dict(fa=fa, fw=fw, w=wcodes, sw=sw_vec.contiguous().to(device),
+                          sw_cs=1 if sw_vec.numel() > 1 else 0, bounds=bounds, N=N, K=K)
+        return self._plan
+
+    def forward_fused(self, x: torch.Tensor, bias=None) -> torch.Tensor:
+        """Final (..., out) result in ``x.dtype``: quantise + segmented GEMM with
+        de-quantisation and bias fused.  Equivalent to ``forward`` followed by
+        the recombination of ``SegmentLinear.forward``, with the partial sums of
+        input segments combined in fp32 and rounded once."""
+        plan = self._plan or self._build_plan(x.device)
+        K, N = plan["K"], plan["N"]
+        x2 = x.reshape(-1, K)
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        M = x2.shape[0]
+        S = self.chunks if self.seg_mode == "input" else 1
+        bounds = plan["bounds"]
+        dyn = bool(self.input_calibrators[0].dynamic)
+        dual = self.dual_scale
+        if dyn:
+            if self.input_calibrators[0].axis is None:
+                raise NotImplementedError("dynamic activation scales are per token (axis=-1) on the kernel path")
+            pos = torch.empty((S, M), dtype=torch.float32, device=x.device)
+            neg = torch.empty_like(pos) if dual else None
+            per_tok = True
+        else:
+            if "sx" not in plan:
+                def stack(attr):
+                    vals = []
+                    for c, d in zip(self.input_calibrators, self.dual_segments):
+                        vals.append(_as_f32(getattr(c, attr if d else "scale"), x.device).reshape(-1))
+                    return torch.stack(vals)
+                plan["sx"] = (stack("pos_scale"), stack("neg_scale")) if dual else (stack("scale"), None)
+            pos, neg = plan["sx"]  # (S, 1) per segment or (S, M) per token
+            per_tok = pos.shape[-1] > 1
+            if per_tok and pos.shape[-1] != M:
+                raise RuntimeError(f"static per-token scales were calibrated for {pos.shape[-1]} tokens, got {M}")
+        kstride = M if per_tok else 1
+        mask = sum(1 << i for i, d in enumerate(self.dual_segments) if d)
+        codes = ops.quantize(x2, plan["fa"], pos, neg, row_stride=1 if per_tok else 0,
+                             kseg_bounds=bounds if S > 1 else None, kseg_stride=kstride, dual=dual,
+                             dual_kseg_mask=mask, dynamic=dyn)
+        ranges = []
+        for s in range(S):
+            k0, k1 = bounds[s], bounds[s + 1]
+            rs = 1 if per_tok else 0
+            if dual and self.dual_segments[s]:
+                ranges.append(ops.Range(k0, k1 - k0, pos[s], plan["sw"], 2, rs, plan["sw_cs"]))
+                ranges.append(ops.Range(k0, k1 - k0, neg[s], plan["sw"], 3, rs, plan["sw_cs"]))
+            else:
+                ranges.append(ops.Range(k0, k1 - k0, pos[s], plan["sw"], 0, rs, plan["sw_cs"]))
+        ldb = K // 2 if plan["fw"] == ops.FMT_INT4 else K
+        out = ops.gemm(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
+                       lda=K, ldb=ldb, bias=bias)
+        return out.view(*x.shape[:-1], N)

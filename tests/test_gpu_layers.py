@@ -1,0 +1,229 @@
+"""GPU tests of the host-side mirror (SegmentLinear, optimiser, quantize())
+running on the HIP kernels, checked against the CPU oracle.
+
+Every benchmark configuration is run at its real K and N and a reduced M so the
+oracle finishes in seconds; the checks are (a) the exact closed form built from
+the layer's own codes and scales, (b) the path's stated tolerance against the
+fp32 fake-quant linear: 1e-3 relative for integer codes, 1e-2 for e4m3.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import segq_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _np32(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _unpacked_weight_codes(layer, fmt):
+    w = layer.optimizer.weight_manager.weight_tensor.cpu().numpy()
+    if fmt == O.FMT_INT4:
+        return np.stack([O.unpack_int4(r) for r in w])
+    return w
+
+
+def _scale_fn(fmt):
+    bits = 4 if fmt == O.FMT_INT4 else 8
+    if fmt == O.FMT_E4M3:
+        return O.fp8_scale, O.fp8_dual_scales
+    return (lambda a: O.int_scale(a, bits)), (lambda p, n: O.int_dual_scales(p, n, bits))
+
+
+def oracle_layer_output(layer, spec, x_np, out_dtype):
+    """Closed form of the fused forward from the layer's stored codes and scales."""
+    from segquant_amd.workloads import segment_bounds
+    opt = layer.optimizer
+    fa, fw = spec.act, spec.weight
+    wq = _unpacked_weight_codes(layer, fw)
+    N, K = wq.shape
+    M = x_np.shape[0]
+    bounds = segment_bounds(spec)
+    single, dualf = _scale_fn(fa)
+    # weight scale per output column
+    wcals = opt.weight_calibrators
+    if spec.seg_mode == "weight" and len(wcals) > 1:
+        sw = np.concatenate([np.broadcast_to(np.float32(_np32(torch.as_tensor(c.scale))).reshape(-1), (n,)) if
+                             np.ndim(c.scale) == 0 or torch.as_tensor(c.scale).numel() == 1 else
+                             _np32(c.scale) for c, n in zip(wcals, opt.chunksizes)])
+    else:
+        s0 = torch.as_tensor(wcals[0].scale).float().cpu().numpy().reshape(-1)
+        sw = np.broadcast_to(s0, (N,)) if s0.size == 1 else s0
+    sw = sw.astype(np.float32).reshape(1, N)
+    y = np.zeros((M, N), dtype=np.float64)
+    for s in range(len(bounds) - 1):
+        k0, k1 = bounds[s], bounds[s + 1]
+        xs = x_np[:, k0:k1]
+        cal = opt.input_calibrators[s if spec.seg_mode == "input" else 0]
+        dual = opt.dual_segments[s if spec.seg_mode == "input" else 0]
+        if spec.dynamic:
+            if dual:
+                ps, ns = dualf(*O.dual_amax(xs, axis=-1))
+            else:
+                ps = single(np.abs(xs).max(axis=-1))
+        else:
+            if dual:
+                ps, ns = (np.float32(_np32(torch.as_tensor(t))) for t in (cal.pos_scale, cal.neg_scale))
+            else:
+                ps = np.float32(_np32(torch.as_tensor(cal.scale)))
+        ps = np.float32(ps).reshape(-1)
+        psb = ps.reshape(-1, 1) if ps.size > 1 else ps.reshape(1, 1)
+        if dual:
+            ns = np.float32(ns).reshape(-1)
+            nsb = ns.reshape(-1, 1) if ns.size > 1 else ns.reshape(1, 1)
+            cp, cn = O.quantize_act_dual(xs[None], ps if ps.size > 1 else ps[:1], ns if ns.size > 1 else ns[:1], fa)
+            y += O.gemm_acc(cp[0], wq[:, k0:k1], fa, fw) / (psb.astype(np.float64) * sw)
+            y += O.gemm_acc(cn[0], wq[:, k0:k1], fa, fw) / (nsb.astype(np.float64) * sw)
+        else:
+            c = O.quantize_act(xs[None], ps if ps.size > 1 else ps[:1], fa)
+            y += O.gemm_acc(c[0], wq[:, k0:k1], fa, fw) / (psb.astype(np.float64) * sw)
+    if layer.bias:
+        y += _np32(layer.bias_data).astype(np.float64)
+    return y
+
+
+CASES = [(1, 96), (2, 160), (3, 130), (4, 144), (5, 100)]
+
+
+@pytest.mark.parametrize("config,M", CASES)
+def test_benchmark_configs_fused_forward(config, M):
+    from segquant_amd import workloads as W
+    seen = set()
+    for spec in W.config_linears(config, M=M):
+        if (spec.name.split("_m")[0], spec.K, spec.N) in seen:
+            continue
+        seen.add((spec.name.split("_m")[0], spec.K, spec.N))
+        layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+        assert layer.optimizer.real_quant, spec.name
+        xin = x.to(spec.x_dtype).to(DEV)
+        out = layer(xin)
+        assert out.shape == (M, spec.N) and out.dtype == spec.x_dtype
+        got = _np32(out).astype(np.float64)
+        x_np = _np32(xin)
+        want = oracle_layer_output(layer, spec, x_np, spec.x_dtype)
+        scale = np.abs(want).max()
+        fp8 = spec.act == O.FMT_E4M3
+        tol = {torch.float32: 3e-6, torch.bfloat16: 2.0 ** -8}[spec.x_dtype] + (1e-3 if fp8 else 0.0)
+        assert np.abs(got - want).max() <= tol * scale, (spec.name, np.abs(got - want).max() / scale)
+        # (b) fp32 input through the same layer vs the fp32 fake-quant linear
+        layer_f, _ = W.build_layer(spec, device=DEV, real_quant=False, x=x)
+        ref = _np32(layer_f(x.to(DEV))).astype(np.float64)
+        real32 = _np32(layer(x.to(DEV))).astype(np.float64)
+        rel = np.abs(real32 - ref).max() / np.abs(ref).max()
+        assert rel <= (1e-2 if fp8 else 1e-3), (spec.name, rel)
+
+
+@pytest.mark.parametrize("kernel", ["Wint8Aint8", "Wfpe4m3Afpe4m3", "Wint4Aint8"])
+@pytest.mark.parametrize("seg_mode", ["weight", "input"])
+@pytest.mark.parametrize("axis", [False, True])
+@pytest.mark.parametrize("dual", [False, True])
+def test_chunked_route_matches_fused_route(kernel, seg_mode, axis, dual):
+    """forward(chunked=True) goes through the reference-convention operator
+    registered in ext_dict; recombining its output must give the fused result."""
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    w_t, a_t = kernel[1:].split("A")
+    M, K, N, S = 24, 256, 192, 2
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(M, K, generator=g)
+    if dual:
+        x = torch.nn.functional.silu(x * 2)
+    lin = torch.nn.Linear(K, N)
+    layer = SegmentLinear(K, N, bias=True, seg_mode=seg_mode, chunks=S, custom_weight_tensor=lin.weight.data,
+                          custom_bias_tensor=lin.bias.data, input_quant_type=a_t, weight_quant_type=w_t,
+                          input_quant_args={"real_quant": True, "dual_scale": dual, "axis": -1 if axis else None},
+                          weight_quant_args={"real_quant": True, "axis": 1 if axis else None}, device=DEV)
+    xd = x.to(DEV)
+    layer.calibrate(xd)
+    layer.finish_calibrate()
+    fused = layer(xd)
+    chunks = layer(xd, chunked=True)
+    assert chunks.shape[0] == S
+    if seg_mode == "weight":
+        rec = chunks.movedim(0, -2).reshape(M, -1)
+    else:
+        rec = chunks.sum(0)
+    rec = rec + layer.bias_data
+    tol = 2e-3 if a_t == "fpe4m3" else 1e-5
+    assert (rec - fused).abs().max().item() <= tol * fused.abs().max().item()
+    ref = lin.to(DEV)(xd)
+    assert ((fused - ref).norm() / ref.norm()).item() < (0.2 if w_t == "int4" else 0.05)
+
+
+class _ChunkModel(torch.nn.Module):
+    """SiLU -> Linear(D, 6D) -> chunk(6): the adaLN pattern of the reference's
+    TestModel (test/test_linear.py:69-92)."""
+
+    def __init__(self, d):
+        super().__init__()
+        self.silu = torch.nn.SiLU()
+        self.linear = torch.nn.Linear(d, 6 * d)
+        self.norm = torch.nn.LayerNorm(d, elementwise_affine=False, eps=1e-6)
+
+    def forward(self, x, emb):
+        shift, scale, gate, *_ = self.linear(self.silu(emb)).chunk(6, dim=1)
+        return self.norm(x) * (1 + scale) + shift, gate
+
+
+class _ConcatModel(torch.nn.Module):
+    """two linears -> cat -> Linear(2D, 3D): the reference's TestInputModel (:94-108)."""
+
+    def __init__(self, d):
+        super().__init__()
+        self.linear_1 = torch.nn.Linear(d, d)
+        self.linear_2 = torch.nn.Linear(d, d)
+        self.linear = torch.nn.Linear(2 * d, 3 * d)
+
+    def forward(self, x, emb):
+        return self.linear(torch.cat([self.linear_1(x), self.linear_2(emb)], dim=1))
+
+
+@pytest.mark.parametrize("atype,wtype", [("INT8", "INT8"), ("FP8E4M3", "FP8E4M3"), ("INT8", "INT4")])
+@pytest.mark.parametrize("axis", [False, True])
+@pytest.mark.parametrize("model_kind", ["chunk", "concat"])
+def test_quantize_real_vs_fake_like_the_reference_grid(atype, wtype, axis, model_kind):
+    """The reference's test_mix_real grid (test/test_linear.py:821-913) with its
+    data recipe (5 calibration batches of rand(3, D), seeds 42 / 1234); it only
+    prints the norms, here fake and real must agree."""
+    import copy
+    from segquant_amd.config import Calibrate, DType, Optimum
+    from segquant_amd.torch.quantization import quantize
+    D = 256
+    torch.manual_seed(0)
+    model = (_ChunkModel(D) if model_kind == "chunk" else _ConcatModel(D)).to(DEV)
+    g = torch.Generator().manual_seed(42)
+    loader = [((torch.rand(3, D, generator=g), torch.rand(3, D, generator=g)),) for _ in range(5)]
+    cfg = {"default": {"enable": True, "seglinear": True, "search_patterns": [], "real_quant": False,
+                       "opt": {"type": Optimum.DEFAULT}, "calib": {"type": Calibrate.AMAX},
+                       "input_quant": {"type": DType[atype], "axis": -1 if axis else None},
+                       "weight_quant": {"type": DType[wtype], "axis": 1 if axis else None}}}
+    segs = ({"linear": {"seg_mode": "weight", "chunks": 6}} if model_kind == "chunk"
+            else {"linear": {"seg_mode": "input", "chunks": 2}})
+    dual = {"linear"} if model_kind == "chunk" else set()
+    fake = quantize(copy.deepcopy(model), loader, copy.deepcopy(cfg), seg_configs=segs, dual_scale_linears=dual)
+    cfg["default"]["real_quant"] = True
+    real = quantize(copy.deepcopy(model), loader, copy.deepcopy(cfg), seg_configs=segs, dual_scale_linears=dual)
+    assert real.linear.optimizer.real_quant and not fake.linear.optimizer.real_quant
+    g = torch.Generator().manual_seed(1234)
+    x, emb = torch.rand(3, D, generator=g).to(DEV), torch.rand(3, D, generator=g).to(DEV)
+    with torch.no_grad():
+        a = model(x, emb)
+        b = fake(x, emb)
+        c = real(x, emb)
+    a, b, c = (t[0] if isinstance(t, tuple) else t for t in (a, b, c))
+    tol = 1e-2 if atype == "FP8E4M3" else 1e-3
+    assert (b - c).abs().max().item() <= tol * b.abs().max().item()
+    assert ((a - c).norm() / a.norm()).item() < (0.25 if wtype == "INT4" else 0.08)
+
+
+def test_unsupported_kernel_type_warns_and_uses_fake_path(capsys):
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    lin = torch.nn.Linear(64, 32)
+    layer = SegmentLinear(64, 32, custom_weight_tensor=lin.weight.data, custom_bias_tensor=lin.bias.data,
+                          input_quant_type="int4", weight_quant_type="int4",
+                          input_quant_args={"real_quant": True}, weight_quant_args={"real_quant": True}, device=DEV)
+    assert "Wint4Aint4" in capsys.readouterr().out
+    assert layer.optimizer.real_quant is False
