@@ -1,6 +1,7 @@
 // C ABI of libsegq: argument checks, kernel selection, launches.
 #include "segq_gemm_kernel.h"
 #include <string.h>
+#include <stdlib.h>
 
 namespace segq {
 
@@ -26,13 +27,21 @@ int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipSt
 static bool is_float_dtype(int t) { return t == SEGQ_F32 || t == SEGQ_F16 || t == SEGQ_BF16; }
 static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// Tile choice when the caller leaves it to the library: 128 x 128 unless that
-// leaves CUs idle, then 64 x 128 (measured on FLUX / SD3 / SDXL shapes).
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold) {
-    (void)fold;
-    const TileCfg& c = TILE_CFGS[2];
-    const int64_t tiles = ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
-    return tiles >= 256 ? 2 : 3;
+// Tile choice when the caller leaves it to the library.  The 8-wave kernel needs
+// K in whole 128-byte steps and 32-bit row offsets; among its tiles take the
+// largest that still gives every CU a workgroup.
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok) {
+    auto tiles = [&](int cfg) {
+        const TileCfg& c = TILE_CFGS[cfg];
+        return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
+    };
+    if (wide_ok) {
+        const int first = FIRST_WIDE_CFG + (fold ? 1 : 0);  // no 256 x 256 with a second accumulator set
+        for (int cfg = first; cfg < FIRST_WIDE_CFG + 4; ++cfg)
+            if (tiles(cfg) >= 256) return cfg;
+        if (tiles(FIRST_WIDE_CFG + 3) >= 128) return FIRST_WIDE_CFG + 3;
+    }
+    return tiles(2) >= 256 ? 2 : 3;
 }
 
 static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
@@ -97,11 +106,21 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     p.bsSx = d->batch_stride_sx; p.bsSw = d->batch_stride_sw;
     p.out_dtype = d->out_dtype; p.bias_dtype = d->bias_dtype;
     p.nr = d->n_ranges;
+    { const char* e = getenv("SEGQ_DBG"); p.dbg = e ? atoi(e) : 0; }
     const bool fold = d->n_ranges > 1;
+    bool wide_ok = d->m * d->lda < (int64_t)1 << 32 && d->n * d->ldb < (int64_t)1 << 32;
+    for (int i = 0; i < d->n_ranges; ++i) wide_ok = wide_ok && d->ranges[i].k_begin % 128 == 0 && d->ranges[i].k_len % 128 == 0;
     int cfg;
-    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold);
+    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok);
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
+    if (cfg >= FIRST_WIDE_CFG) {
+        if (!wide_ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs K ranges in multiples of 128", cfg + 1);
+        if (fold && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
+    } else if (cfg >= FIRST_BIG_CFG) {
+        if (!wide_ok || w4 || fold)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs one range, 8-bit weights and K in multiples of 128", cfg + 1);
+    }
     const TileCfg& c = TILE_CFGS[cfg];
     p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);
     p.tiles_n = (int32_t)((d->n + c.bn - 1) / c.bn);
@@ -109,6 +128,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff || d->batch > 65535) return fail(SEGQ_ERR_ARG, "segq_gemm: grid too large");
     const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
     p.vec_store = ((d->ldo * osz) % (4 * osz) == 0) && ((d->batch_stride_out * osz) % (4 * osz) == 0) && al(d->out, 4 * osz);
+    p.vec_store16 = osz == 2 && d->ldo % 8 == 0 && d->batch_stride_out % 8 == 0 && al(d->out, 16);
     if (i8) return launch_gemm_i8(p, cfg, fold, d->batch, st);
     if (f8) return launch_gemm_f8(p, cfg, fold, d->batch, st);
     return launch_gemm_w4(p, cfg, fold, d->batch, st);

@@ -1,5 +1,5 @@
 // Instances of the segmented GEMM kernel for one operand format.
-#include "segq_gemm_kernel.h"
+#include "segq_gemm_wide.h"
 namespace segq {
 int launch_gemm_f8(const GemmParams& p, int cfg, bool fold, int64_t batch, hipStream_t st) {
     return launch_format<GEMM_F8, false>(p, cfg, fold, batch, st);

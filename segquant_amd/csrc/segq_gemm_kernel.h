@@ -44,17 +44,23 @@ struct GemmParams {
     int32_t out_dtype, bias_dtype;
     int32_t nr;
     int32_t tiles_m, tiles_n, group_m;
-    int32_t vec_store;  // output rows allow 8/16-byte vector stores
+    int32_t vec_store;    // output rows allow 4-element vector stores
+    int32_t vec_store16;  // 16-bit output rows allow 16-byte stores
+    int32_t dbg;
     KRange r[SEGQ_MAX_RANGES];
 };
 
 enum { GEMM_I8 = 0, GEMM_F8 = 1 };
 constexpr int BK = 128;  // code bytes of K per step
 
-// Chunk swizzle: a bijection of 0..7 over any 8 consecutive rows AND over any 8
-// rows of equal parity out of 16, so 16-byte accesses of 8 (32-bank view) or 16
-// (64-bank view) consecutive rows at one logical chunk touch distinct banks.
-__device__ __forceinline__ int swz(int row) { return (((row >> 1) & 3) << 1) | (((row >> 3) ^ row) & 1); }
+// Chunk swizzle.  The LDS of gfx950 has 64 banks of 4 bytes (a 256-byte span),
+// so a 128-byte row covers half of them and rows 2j and 2j+1 cover different
+// halves.  XOR-ing the 16-byte chunk index with (row >> 1) & 7 makes the MFMA
+// fragment reads (16 or 32 consecutive rows at one logical chunk) and the
+// staging writes (8 lanes across one row) free of bank conflicts; measured with
+// a four-wave ds_read_b128 loop: 18 clocks per instruction against 32 for
+// row & 7 on 32-row fragments and 64 without a swizzle.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 // 0xFF in every byte of x whose top bit is set.
 __device__ __forceinline__ uint32_t neg_byte_mask(uint32_t x) { return ((x >> 7) & 0x01010101u) * 0xFFu; }
@@ -304,18 +310,19 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
             kn = (rn < p.nr) ? p.r[rn].k0 : 0;
         }
         const bool more = rn < p.nr;
-        if (more) load_tile(rn, kn);
-        compute(buf);
+        if (more && !(p.dbg & 1)) load_tile(rn, kn);
+        if (!(p.dbg & 2)) compute(buf);
         if (FOLD && range_done) fold(r);
         if (!more) break;
-        store_tile(buf ^ 1, p.r[rn].a_sel);
-        __syncthreads();
+        if (!(p.dbg & 1)) store_tile(buf ^ 1, p.r[rn].a_sel);
+        if (!(p.dbg & 4)) __syncthreads();
         buf ^= 1;
         r = rn;
         k = kn;
     }
 
     // ---- epilogue
+    if (p.dbg & 8) return;
     const int64_t c_off = z * p.bsC;
     if (p.out_dtype == SEGQ_ACC) {
         // raw accumulators of the single range
@@ -389,9 +396,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
 
 // ---- host-side launch of one (format, tile, fold) instance -------------------
 struct TileCfg { int bm, bn, wgm, wgn; };
-constexpr int NUM_TILE_CFG = 5;
+constexpr int NUM_TILE_CFG = 14;
+constexpr int FIRST_BIG_CFG = 8;    // two ids: the 4-wave 256 x 256 kernel (segq_gemm_big.h)
+constexpr int FIRST_WIDE_CFG = 10;  // four ids: the 8-wave kernel (segq_gemm_wide.h)
 constexpr TileCfg TILE_CFGS[NUM_TILE_CFG] = {
     {256, 256, 2, 2}, {256, 128, 2, 2}, {128, 128, 2, 2}, {64, 128, 2, 2}, {128, 256, 2, 2},
+    {256, 256, 2, 4}, {256, 256, 4, 2}, {256, 128, 4, 2}, {256, 256, 2, 2}, {256, 256, 2, 2},
+    {256, 256, 4, 2}, {256, 128, 4, 2}, {128, 256, 2, 4}, {128, 128, 2, 4},
 };
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
@@ -409,8 +420,22 @@ int launch_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     return check_launch("segq_gemm");
 }
 
+template <int FMT, bool DIRECT>
+int launch_big(const GemmParams& p, int64_t batch, hipStream_t st);
+template <int FMT, bool B4>
+int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st);
+
 template <int FMT, bool B4>
 int launch_format(const GemmParams& p, int cfg, bool fold, int64_t batch, hipStream_t st) {
+    if (cfg >= FIRST_WIDE_CFG) {
+        bool asel = false;
+        for (int i = 0; i < p.nr; ++i) asel = asel || p.r[i].a_sel >= 2;
+        return launch_wide<FMT, B4>(p, cfg - FIRST_WIDE_CFG, fold, asel, batch, st);
+    }
+    if constexpr (!B4) {
+        if (!fold && cfg == FIRST_BIG_CFG) return launch_big<FMT, false>(p, batch, st);
+        if (!fold && cfg == FIRST_BIG_CFG + 1) return launch_big<FMT, true>(p, batch, st);
+    }
     switch (cfg * 2 + (fold ? 1 : 0)) {
         case 0: return launch_instance<256, 256, 2, 2, FMT, B4, false>(p, batch, st);
         case 2: return launch_instance<256, 128, 2, 2, FMT, B4, false>(p, batch, st);
@@ -421,6 +446,10 @@ int launch_format(const GemmParams& p, int cfg, bool fold, int64_t batch, hipStr
         case 7: return launch_instance<64, 128, 2, 2, FMT, B4, true>(p, batch, st);
         case 8: return launch_instance<128, 256, 2, 2, FMT, B4, false>(p, batch, st);
         case 9: return launch_instance<128, 256, 2, 2, FMT, B4, true>(p, batch, st);
+        case 10: return launch_instance<256, 256, 2, 4, FMT, B4, false>(p, batch, st);
+        case 12: return launch_instance<256, 256, 4, 2, FMT, B4, false>(p, batch, st);
+        case 14: return launch_instance<256, 128, 4, 2, FMT, B4, false>(p, batch, st);
+        case 15: return launch_instance<256, 128, 4, 2, FMT, B4, true>(p, batch, st);
     }
     return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: no kernel for tile %d%s", cfg + 1, fold ? " with several ranges" : "");
 }

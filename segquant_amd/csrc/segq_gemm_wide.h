@@ -1,0 +1,403 @@
+// Segmented GEMM, main kernel: eight waves per workgroup, K walked in whole
+// 128-byte steps, operands streamed global -> LDS without passing through
+// registers wherever no per-byte transform is needed.
+//
+// Design points, each backed by a measurement on MI355X:
+//  * Two waves per SIMD.  The 4-pass v_mfma_i32_16x16x64_i8 issued back to back
+//    from ONE wave reaches 56 % of the matrix pipe's rate, from two waves 90 %.
+//  * global_load_lds_dwordx4 for plain operands: no staging VGPRs, no ds_write
+//    instructions (ds_write_b128 moves ~80 B/clk/CU, a third of what reads do),
+//    and nothing in the loop consumes a loaded value, so the loads of step k+1
+//    really overlap the MFMAs of step k.  The LDS side of such a load is
+//    lane-linear, so the bank swizzle is applied to the global address instead.
+//  * Activations that need sign selection (merged DualScale codes) and int4
+//    weights go through registers; their transform is branch-free.
+//  * Epilogue through LDS for 16-bit outputs: each lane owns 4 consecutive
+//    columns of 16 different rows, which as direct stores are 32-byte pieces of
+//    16 lines per instruction (measured 1.7 TB/s); transposed through a private
+//    LDS patch every store instruction writes four full 256-byte row pieces.
+#pragma once
+#include "segq_gemm_big.h"
+
+namespace segq {
+
+template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmParams p) {
+    constexpr int NW = WGM * WGN, NT = NW * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 16, TN = WN / 16;
+    constexpr int A_IT = BM * 8 / NT;                 // 16-byte chunks per thread, activations
+    constexpr int B_IT = (B4 ? BN * 4 : BN * 8) / NT;  // same, weights (packed chunks when int4)
+    constexpr int RPI = NT / 8;                        // rows covered by one pass of all threads
+    constexpr int RPI4 = NT / 4;
+    static_assert(BM * 8 % NT == 0 && BN * 4 % NT == 0 && RPI % 16 == 0, "tile does not divide over the threads");
+    static_assert(!B4 || FMT == GEMM_I8, "int4 weights pair with int8 activations");
+    typedef typename AccT<FMT>::type acc_t;
+    typedef typename AccT<FMT>::elem acc_e;
+    const acc_t acc_zero = {0, 0, 0, 0};
+
+    extern __shared__ __align__(16) uint8_t smem[];
+    uint8_t* const As = smem;                // [2][BM][128]
+    uint8_t* const Bs = smem + 2 * BM * BK;  // [2][BN][128]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int lrow = lane & 15, lgrp = lane >> 4;
+
+    int bid = blockIdx.x;
+    {
+        const int nb = p.tiles_m * p.tiles_n;
+        if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+    }
+    int tile_m, tile_n;
+    {
+        const int gsz = p.group_m * p.tiles_n;
+        const int g = bid / gsz;
+        const int first_m = g * p.group_m;
+        const int rows_in_group = min(p.tiles_m - first_m, p.group_m);
+        const int in_g = bid - g * gsz;
+        tile_m = first_m + in_g % rows_in_group;
+        tile_n = in_g / rows_in_group;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int64_t z = blockIdx.y;
+    const uint8_t* const Ab = p.A + z * p.bsA;
+    const uint8_t* const A2b = p.A2 ? p.A2 + z * p.bsA : nullptr;
+    const uint8_t* const Bb = p.B + z * p.bsB;
+
+    // ---- staging.  Thread t, pass i: row i * RPI + t / 8, physical chunk t % 8,
+    // which holds logical chunk (t % 8) ^ swz(row).
+    const int s_row = tid >> 3;
+    const int s_pc = tid & 7;
+    const int s_lc = s_pc ^ swz(s_row);
+    uint32_t a_goff[A_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) a_goff[i] = (uint32_t)min(m0 + s_row + i * RPI, p.M - 1) * (uint32_t)p.lda + s_lc * 16;
+    // weights: same scheme, or 4 packed chunks per row when int4
+    const int b_row = B4 ? (tid >> 2) : s_row;
+    const int b_pk = tid & 3;  // int4: packed chunk = 32 k = logical chunks 2 b_pk, 2 b_pk + 1
+    constexpr int B_RSTEP = B4 ? RPI4 : RPI;
+    uint32_t b_goff[B_IT];
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i)
+        b_goff[i] = (uint32_t)min(n0 + b_row + i * B_RSTEP, p.N - 1) * (uint32_t)p.ldb + (B4 ? b_pk : s_lc) * 16;
+    const int b_sw = swz(b_row);
+    const int w_lds = wave * 8 * BK;  // direct loads: the 8 rows this wave fills per pass
+
+    uint4 ra[ASEL ? A_IT : 1], rb[B4 ? B_IT : 1];
+
+    auto issue_loads = [&](const uint8_t* ap, int k, int buf) {
+        if constexpr (ASEL) {
+#pragma unroll
+            for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const uint4*>(ap + k + a_goff[i]);
+        } else {
+            uint8_t* as = As + buf * BM * BK + w_lds;
+#pragma unroll
+            for (int i = 0; i < A_IT; ++i) load16_to_lds(ap + k + a_goff[i], as + i * RPI * BK);
+        }
+        if constexpr (B4) {
+#pragma unroll
+            for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const uint4*>(Bb + (k >> 1) + b_goff[i]);
+        } else {
+            uint8_t* bs = Bs + buf * BN * BK + w_lds;
+#pragma unroll
+            for (int i = 0; i < B_IT; ++i) load16_to_lds(Bb + k + b_goff[i], bs + i * RPI * BK);
+        }
+    };
+    // sel_or / sel_xor: branch-free sign selection, kept = x & ((negmask ^ sel_xor) | sel_or)
+    auto commit_loads = [&](int buf, uint32_t sel_or, uint32_t sel_xor) {
+        if constexpr (ASEL) {
+            uint8_t* as = As + buf * BM * BK + s_row * BK + s_pc * 16;
+#pragma unroll
+            for (int i = 0; i < A_IT; ++i) {
+                uint4 v = ra[i];
+                v.x &= (neg_byte_mask(v.x) ^ sel_xor) | sel_or;
+                v.y &= (neg_byte_mask(v.y) ^ sel_xor) | sel_or;
+                v.z &= (neg_byte_mask(v.z) ^ sel_xor) | sel_or;
+                v.w &= (neg_byte_mask(v.w) ^ sel_xor) | sel_or;
+                *reinterpret_cast<uint4*>(as + i * RPI * BK) = v;
+            }
+        }
+        if constexpr (B4) {
+            uint8_t* bs = Bs + buf * BN * BK + b_row * BK;
+#pragma unroll
+            for (int i = 0; i < B_IT; ++i) {
+                uint4 lo, hi;
+                unpack8_i4x16(rb[i].x, lo.x, lo.y);
+                unpack8_i4x16(rb[i].y, lo.z, lo.w);
+                unpack8_i4x16(rb[i].z, hi.x, hi.y);
+                unpack8_i4x16(rb[i].w, hi.z, hi.w);
+                uint8_t* row = bs + i * B_RSTEP * BK;
+                *reinterpret_cast<uint4*>(row + (((2 * b_pk) ^ b_sw) << 4)) = lo;
+                *reinterpret_cast<uint4*>(row + (((2 * b_pk + 1) ^ b_sw) << 4)) = hi;
+            }
+        }
+        if constexpr (!ASEL || !B4) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): direct loads have landed
+    };
+
+    acc_t acc[TN][TM];
+    v4f accf[FOLD ? TN : 1][FOLD ? TM : 1];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b) acc[a][b] = acc_zero;
+    if constexpr (FOLD) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) accf[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int f_sw = swz(lrow);
+    const int a_frag = (wm * WM + lrow) * BK;
+    const int b_frag = (wn * WN + lrow) * BK;
+
+    auto compute = [&](int buf) {
+        const uint8_t* as = As + buf * BM * BK + a_frag;
+        const uint8_t* bs = Bs + buf * BN * BK + b_frag;
+        if constexpr (FMT == GEMM_I8) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int off = ((ks * 4 + lgrp) ^ f_sw) << 4;
+                v4i fa[TM], fb[TN];
+#pragma unroll
+                for (int t = 0; t < TM; ++t) fa[t] = *reinterpret_cast<const v4i*>(as + t * 16 * BK + off);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) fb[t] = *reinterpret_cast<const v4i*>(bs + t * 16 * BK + off);
+#pragma unroll
+                for (int a = 0; a < TN; ++a)
+#pragma unroll
+                    for (int b = 0; b < TM; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[a], fa[b], acc[a][b], 0, 0, 0);
+            }
+        } else {
+            const int off0 = ((2 * lgrp) ^ f_sw) << 4;
+            const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
+            v8i fa[TM], fb[TN];
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const v4i lo = *reinterpret_cast<const v4i*>(as + t * 16 * BK + off0);
+                const v4i hi = *reinterpret_cast<const v4i*>(as + t * 16 * BK + off1);
+                fa[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const v4i lo = *reinterpret_cast<const v4i*>(bs + t * 16 * BK + off0);
+                const v4i hi = *reinterpret_cast<const v4i*>(bs + t * 16 * BK + off1);
+                fb[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[a], fa[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+        }
+    };
+
+    // lane's output coordinates: row m_base + 16 b, columns n_base + 16 a + 0..3
+    const int m_base = m0 + wm * WM + lrow;
+    const int n_base = n0 + wn * WN + 4 * lgrp;
+
+    auto range_rx = [&](int r, float (&rx)[TM]) {
+        const float* sx = p.r[r].sx + z * p.bsSx;
+        const int rs = p.r[r].sx_rs;
+#pragma unroll
+        for (int b = 0; b < TM; ++b) rx[b] = 1.0f / sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs];
+    };
+    auto range_rw = [&](int r, int a, float (&rw)[4]) {
+        const float* sw = p.r[r].sw + z * p.bsSw;
+        const int cs = p.r[r].sw_cs;
+        const float unscale = B4 ? 0.0625f : 1.0f;  // the staged int4 weights carry an exact factor 16
+#pragma unroll
+        for (int v = 0; v < 4; ++v) rw[v] = unscale / sw[(int64_t)min(n_base + a * 16 + v, p.N - 1) * cs];
+    };
+    auto fold = [&](int r) {
+        if constexpr (FOLD) {
+            float rx[TM];
+            range_rx(r, rx);
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                float rw[4];
+                range_rw(r, a, rw);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) accf[a][b][v] += (float)acc[a][b][v] * rx[b] * rw[v];
+                    acc[a][b] = acc_zero;
+                }
+            }
+        }
+    };
+    auto sel_masks = [&](int a_sel, uint32_t& so, uint32_t& sx) {
+        so = (a_sel >= 2) ? 0u : 0xFFFFFFFFu;
+        sx = (a_sel == 2) ? 0xFFFFFFFFu : 0u;
+    };
+
+    // ---- main loop over (range, k) steps; every range is whole 128-byte steps
+    int r = 0, k = p.r[0].k0;
+    uint32_t so, sxm;
+    sel_masks(p.r[0].a_sel, so, sxm);
+    issue_loads((p.r[0].a_sel == 1) ? A2b : Ab, k, 0);
+    commit_loads(0, so, sxm);
+    __syncthreads();
+    int buf = 0;
+    while (true) {
+        int rn = r, kn = k + BK;
+        const bool range_done = kn >= p.r[r].k1;
+        if (range_done) {
+            rn = r + 1;
+            kn = (rn < p.nr) ? p.r[rn].k0 : 0;
+        }
+        const bool more = rn < p.nr;
+        if (more) {
+            const int sel = p.r[rn].a_sel;
+            sel_masks(sel, so, sxm);
+            issue_loads((sel == 1) ? A2b : Ab, kn, buf ^ 1);
+        }
+        compute(buf);
+        if (FOLD && range_done) fold(r);
+        if (!more) break;
+        commit_loads(buf ^ 1, so, sxm);
+        __syncthreads();
+        buf ^= 1;
+        r = rn;
+        k = kn;
+    }
+
+    // ---- epilogue
+    const int64_t c_off = z * p.bsC;
+    if (p.out_dtype == SEGQ_ACC) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int m = m_base + b * 16, n = n_base + a * 16;
+                if (m >= p.M) continue;
+                acc_t t = acc[a][b];
+                if constexpr (B4) { t[0] >>= 4; t[1] >>= 4; t[2] >>= 4; t[3] >>= 4; }
+                acc_e* dst = static_cast<acc_e*>(p.C) + c_off + (int64_t)m * p.ldc + n;
+                if (p.vec_store && n + 3 < p.N) {
+                    *reinterpret_cast<acc_t*>(dst) = t;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (n + v < p.N) dst[v] = t[v];
+                }
+            }
+        return;
+    }
+
+    float rx[TM];
+    if constexpr (!FOLD) range_rx(0, rx);
+    const bool is16 = p.out_dtype != SEGQ_F32;
+    const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
+    if (via_lds) {
+        // every wave transposes 16 rows at a time through its own patch of LDS
+        constexpr int RS = WN * 2 + 16;  // row stride in bytes; the 16 spreads rows over the banks
+        __syncthreads();                 // the operand tiles are dead from here on
+        uint8_t* patch = smem + wave * 16 * RS;
+        const int rd_row = lane / (WN / 8), rd_col = lane % (WN / 8);
+        constexpr int ROWS_PER_RD = 64 / (WN / 8);
+        float rwv[TN][4], bvv[TN][4];
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            if constexpr (!FOLD) range_rw(0, a, rwv[a]);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
+        }
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                uint32_t h[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float o = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
+                    h[v] = (p.out_dtype == SEGQ_BF16) ? f32_to_bf16_bits(o) : f32_to_f16_bits(o);
+                }
+                *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
+                    make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < 16 / ROWS_PER_RD; ++j) {
+                const int row = j * ROWS_PER_RD + rd_row;
+                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + rd_col * 16);
+                const int m = m0 + wm * WM + b * 16 + row;
+                if (m < p.M)
+                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + rd_col * 8) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
+#pragma unroll
+    for (int a = 0; a < TN; ++a) {
+        float rw[4];
+        if constexpr (!FOLD) range_rw(0, a, rw);
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) bv[v] = load_bias(p.bias, p.bias_dtype, min(n_base + a * 16 + v, p.N - 1));
+        }
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int m = m_base + b * 16, n = n_base + a * 16;
+            if (m >= p.M || n >= p.N) continue;
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
+                else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
+            }
+            const int64_t e = c_off + (int64_t)m * p.ldc + n;
+            const bool vec = p.vec_store && (n + 3 < p.N);
+            if (p.out_dtype == SEGQ_F32) store4<SEGQ_F32>(p.C, e, o, vec, p.N - n);
+            else if (p.out_dtype == SEGQ_BF16) store4<SEGQ_BF16>(p.C, e, o, vec, p.N - n);
+            else store4<SEGQ_F16>(p.C, e, o, vec, p.N - n);
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
+int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
+    auto kern = gemm_wide_kernel<BM, BN, WGM, WGN, FMT, B4, FOLD, ASEL>;
+    constexpr int lds = 2 * (BM + BN) * BK;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", lds);
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    hipLaunchKernelGGL(kern, grid, dim3(WGM * WGN * 64), lds, st, p);
+    return check_launch("segq_gemm");
+}
+
+// wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
+template <int FMT, bool B4>
+int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st) {
+#define SEGQ_WIDE(BM_, BN_, WGM_, WGN_, FOLD_)                                                          \
+    return asel ? launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, true>(p, batch, st)       \
+                : launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, false>(p, batch, st)
+    if (!fold) {
+        switch (wcfg) {
+            case 0: SEGQ_WIDE(256, 256, 4, 2, false);
+            case 1: SEGQ_WIDE(256, 128, 4, 2, false);
+            case 2: SEGQ_WIDE(128, 256, 2, 4, false);
+            case 3: SEGQ_WIDE(128, 128, 2, 4, false);
+        }
+    } else {
+        switch (wcfg) {  // a second accumulator set: halve the wave tile
+            case 0: case 1: SEGQ_WIDE(256, 128, 4, 2, true);
+            case 2: SEGQ_WIDE(128, 256, 2, 4, true);
+            case 3: SEGQ_WIDE(128, 128, 2, 4, true);
+        }
+    }
+#undef SEGQ_WIDE
+    return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: no wide kernel %d", wcfg);
+}
+
+}  // namespace segq
