@@ -1,7 +1,6 @@
 // C ABI of libsegq: argument checks, kernel selection, launches.
 #include "segq_gemm_kernel.h"
 #include <string.h>
-#include <stdlib.h>
 
 namespace segq {
 
@@ -106,7 +105,6 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     p.bsSx = d->batch_stride_sx; p.bsSw = d->batch_stride_sw;
     p.out_dtype = d->out_dtype; p.bias_dtype = d->bias_dtype;
     p.nr = d->n_ranges;
-    { const char* e = getenv("SEGQ_DBG"); p.dbg = e ? atoi(e) : 0; }
     const bool fold = d->n_ranges > 1;
     bool wide_ok = d->m * d->lda < (int64_t)1 << 32 && d->n * d->ldb < (int64_t)1 << 32;
     for (int i = 0; i < d->n_ranges; ++i) wide_ok = wide_ok && d->ranges[i].k_begin % 128 == 0 && d->ranges[i].k_len % 128 == 0;

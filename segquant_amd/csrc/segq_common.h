@@ -37,4 +37,17 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
     return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two fp32 values rounded to nearest even and packed, a in the low half
+// (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t));
+}
+__device__ __forceinline__ uint32_t pack2_f16(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, f16x2_t));
+}
+
 }  // namespace segq

@@ -53,13 +53,13 @@ __device__ __forceinline__ void store4(void* C, int64_t e, const float (&o)[4], 
                 if (v < n_left) dst[v] = o[v];
         }
     } else {
-        uint32_t h[4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) h[v] = (OUT == SEGQ_BF16) ? f32_to_bf16_bits(o[v]) : f32_to_f16_bits(o[v]);
+        const uint32_t lo = (OUT == SEGQ_BF16) ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]);
+        const uint32_t hi = (OUT == SEGQ_BF16) ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]);
         uint16_t* dst = static_cast<uint16_t*>(C) + e;
         if (vec) {
-            *reinterpret_cast<uint2*>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+            *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
         } else {
+            const uint32_t h[4] = {lo & 0xffffu, lo >> 16, hi & 0xffffu, hi >> 16};
 #pragma unroll
             for (int v = 0; v < 4; ++v)
                 if (v < n_left) dst[v] = (uint16_t)h[v];

@@ -46,7 +46,6 @@ struct GemmParams {
     int32_t tiles_m, tiles_n, group_m;
     int32_t vec_store;    // output rows allow 4-element vector stores
     int32_t vec_store16;  // 16-bit output rows allow 16-byte stores
-    int32_t dbg;
     KRange r[SEGQ_MAX_RANGES];
 };
 
@@ -310,19 +309,18 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
             kn = (rn < p.nr) ? p.r[rn].k0 : 0;
         }
         const bool more = rn < p.nr;
-        if (more && !(p.dbg & 1)) load_tile(rn, kn);
-        if (!(p.dbg & 2)) compute(buf);
+        if (more) load_tile(rn, kn);
+        compute(buf);
         if (FOLD && range_done) fold(r);
         if (!more) break;
-        if (!(p.dbg & 1)) store_tile(buf ^ 1, p.r[rn].a_sel);
-        if (!(p.dbg & 4)) __syncthreads();
+        store_tile(buf ^ 1, p.r[rn].a_sel);
+        __syncthreads();
         buf ^= 1;
         r = rn;
         k = kn;
     }
 
     // ---- epilogue
-    if (p.dbg & 8) return;
     const int64_t c_off = z * p.bsC;
     if (p.out_dtype == SEGQ_ACC) {
         // raw accumulators of the single range

@@ -21,6 +21,127 @@
 
 namespace segq {
 
+// Scale, add bias, round once, store.  16-bit outputs of full tiles go through a
+// per-wave LDS patch so that every store instruction writes whole row pieces.
+template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
+__device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT<FMT>::type (&acc)[BN / WGN / 16][BM / WGM / 16],
+                                              v4f (&accf)[FOLD ? BN / WGN / 16 : 1][FOLD ? BM / WGM / 16 : 1],
+                                              uint8_t* smem, int64_t z, int m0, int n0, int wave, int lane) {
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 16, TN = WN / 16;
+    typedef typename AccT<FMT>::type acc_t;
+    typedef typename AccT<FMT>::elem acc_e;
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    const int m_base = m0 + wm * WM + lrow;
+    const int n_base = n0 + wn * WN + 4 * lgrp;
+    auto range_rx = [&](int r, float (&rx)[TM]) {
+        const float* sx = p.r[r].sx + z * p.bsSx;
+        const int rs = p.r[r].sx_rs;
+#pragma unroll
+        for (int b = 0; b < TM; ++b) rx[b] = __builtin_amdgcn_rcpf(sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs]);
+    };
+    auto range_rw = [&](int r, int a, float (&rw)[4]) {
+        const float* sw = p.r[r].sw + z * p.bsSw;
+        const int cs = p.r[r].sw_cs;
+        const float unscale = B4 ? 0.0625f : 1.0f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) rw[v] = unscale * __builtin_amdgcn_rcpf(sw[(int64_t)min(n_base + a * 16 + v, p.N - 1) * cs]);
+    };
+    const int64_t c_off = z * p.bsC;
+    if (p.out_dtype == SEGQ_ACC) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int m = m_base + b * 16, n = n_base + a * 16;
+                if (m >= p.M) continue;
+                acc_t t = acc[a][b];
+                if constexpr (B4) { t[0] >>= 4; t[1] >>= 4; t[2] >>= 4; t[3] >>= 4; }
+                acc_e* dst = static_cast<acc_e*>(p.C) + c_off + (int64_t)m * p.ldc + n;
+                if (p.vec_store && n + 3 < p.N) {
+                    *reinterpret_cast<acc_t*>(dst) = t;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (n + v < p.N) dst[v] = t[v];
+                }
+            }
+        return;
+    }
+
+    float rx[TM];
+    if constexpr (!FOLD) range_rx(0, rx);
+    const bool is16 = p.out_dtype != SEGQ_F32;
+    const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
+    if (via_lds) {
+        // every wave transposes 16 rows at a time through its own patch of LDS
+        constexpr int RS = WN * 2 + 16;  // row stride in bytes; the 16 spreads rows over the banks
+        __syncthreads();                 // the operand tiles are dead from here on
+        uint8_t* patch = smem + wave * 16 * RS;
+        const int rd_row = lane / (WN / 8), rd_col = lane % (WN / 8);
+        constexpr int ROWS_PER_RD = 64 / (WN / 8);
+        float rwv[TN][4], bvv[TN][4];
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            if constexpr (!FOLD) range_rw(0, a, rwv[a]);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
+        }
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                float o[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    o[v] = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
+                const bool bf = p.out_dtype == SEGQ_BF16;
+                *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
+                    make_uint2(bf ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]),
+                               bf ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]));
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < 16 / ROWS_PER_RD; ++j) {
+                const int row = j * ROWS_PER_RD + rd_row;
+                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + rd_col * 16);
+                const int m = m0 + wm * WM + b * 16 + row;
+                if (m < p.M)
+                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + rd_col * 8) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
+#pragma unroll
+    for (int a = 0; a < TN; ++a) {
+        float rw[4];
+        if constexpr (!FOLD) range_rw(0, a, rw);
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) bv[v] = load_bias(p.bias, p.bias_dtype, min(n_base + a * 16 + v, p.N - 1));
+        }
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int m = m_base + b * 16, n = n_base + a * 16;
+            if (m >= p.M || n >= p.N) continue;
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
+                else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
+            }
+            const int64_t e = c_off + (int64_t)m * p.ldc + n;
+            const bool vec = p.vec_store && (n + 3 < p.N);
+            if (p.out_dtype == SEGQ_F32) store4<SEGQ_F32>(p.C, e, o, vec, p.N - n);
+            else if (p.out_dtype == SEGQ_BF16) store4<SEGQ_BF16>(p.C, e, o, vec, p.N - n);
+            else store4<SEGQ_F16>(p.C, e, o, vec, p.N - n);
+        }
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmParams p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
@@ -204,14 +325,14 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
         const float* sx = p.r[r].sx + z * p.bsSx;
         const int rs = p.r[r].sx_rs;
 #pragma unroll
-        for (int b = 0; b < TM; ++b) rx[b] = 1.0f / sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs];
+        for (int b = 0; b < TM; ++b) rx[b] = __builtin_amdgcn_rcpf(sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs]);
     };
     auto range_rw = [&](int r, int a, float (&rw)[4]) {
         const float* sw = p.r[r].sw + z * p.bsSw;
         const int cs = p.r[r].sw_cs;
         const float unscale = B4 ? 0.0625f : 1.0f;  // the staged int4 weights carry an exact factor 16
 #pragma unroll
-        for (int v = 0; v < 4; ++v) rw[v] = unscale / sw[(int64_t)min(n_base + a * 16 + v, p.N - 1) * cs];
+        for (int v = 0; v < 4; ++v) rw[v] = unscale * __builtin_amdgcn_rcpf(sw[(int64_t)min(n_base + a * 16 + v, p.N - 1) * cs]);
     };
     auto fold = [&](int r) {
         if constexpr (FOLD) {
@@ -266,99 +387,209 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
         k = kn;
     }
 
-    // ---- epilogue
-    const int64_t c_off = z * p.bsC;
-    if (p.out_dtype == SEGQ_ACC) {
+    wide_epilogue<BM, BN, WGM, WGN, FMT, B4, FOLD>(p, acc, accf, smem, z, m0, n0, wave, lane);
+}
+
+// Software-pipelined variant for plain int8 operands (both straight to LDS) with
+// NS LDS stages.  Two stages are what is instantiated: on FLUX shapes three and
+// four stages measured slower (they cost a co-resident workgroup or buy nothing,
+// the global -> LDS path being throughput- rather than latency-bound: ~31 of a
+// measured ~55 B/clk/CU).  The K step is split at its one barrier:
+//
+//   barrier (tile s landed, tile s-1 fully in registers)
+//     DMA tile s+1 into the buffer of tile s-1      <- a whole step of latency cover
+//     LDS -> fragments F0 of tile s
+//     MFMAs on fragments F1 of tile s-1             <- hides the F0 reads
+//     LDS -> fragments F1 of tile s
+//     MFMAs on F0 of tile s                         <- hides the F1 reads
+//   wait own DMA and LDS reads, barrier
+//
+// so fragment reads never stand between an MFMA group and the one before it.
+// s_waitcnt immediate for "vmcnt(n) lgkmcnt(0)" on gfx9-family encodings
+constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }
+
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmParams p) {
+    constexpr int NW = WGM * WGN, NT = NW * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 16, TN = WN / 16;
+    constexpr int A_IT = BM * 8 / NT, B_IT = BN * 8 / NT;
+    constexpr int RPI = NT / 8;
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0 && RPI % 16 == 0, "tile does not divide over the threads");
+    typedef typename AccT<FMT>::type acc_t;
+    static_assert(FMT == GEMM_I8, "two fragment sets per step: the 64-byte int8 MFMA");
+    typedef v4i frag_t;
+    const acc_t acc_zero = {0, 0, 0, 0};
+
+    static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
+    extern __shared__ __align__(16) uint8_t smem[];
+    uint8_t* const As = smem;                  // [NS][BM][128]
+    uint8_t* const Bs = smem + NS * BM * BK;   // [NS][BN][128]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int lrow = lane & 15, lgrp = lane >> 4;
+
+    int bid = blockIdx.x;
+    {
+        const int nb = p.tiles_m * p.tiles_n;
+        if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+    }
+    int tile_m, tile_n;
+    {
+        const int gsz = p.group_m * p.tiles_n;
+        const int g = bid / gsz;
+        const int first_m = g * p.group_m;
+        const int rows_in_group = min(p.tiles_m - first_m, p.group_m);
+        const int in_g = bid - g * gsz;
+        tile_m = first_m + in_g % rows_in_group;
+        tile_n = in_g / rows_in_group;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int64_t z = blockIdx.y;
+    const uint8_t* const Ab = p.A + z * p.bsA;
+    const uint8_t* const A2b = p.A2 ? p.A2 + z * p.bsA : nullptr;
+    const uint8_t* const Bb = p.B + z * p.bsB;
+
+    const int s_row = tid >> 3;
+    const int s_lc = (tid & 7) ^ swz(s_row);
+    uint32_t a_goff[A_IT], b_goff[B_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) a_goff[i] = (uint32_t)min(m0 + s_row + i * RPI, p.M - 1) * (uint32_t)p.lda + s_lc * 16;
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) b_goff[i] = (uint32_t)min(n0 + s_row + i * RPI, p.N - 1) * (uint32_t)p.ldb + s_lc * 16;
+    const int w_lds = wave * 8 * BK;
+
+    auto dma = [&](int r, int k, int buf) {
+        const uint8_t* ap = ((p.r[r].a_sel == 1) ? A2b : Ab) + k;
+        const uint8_t* bp = Bb + k;
+        uint8_t* as = As + buf * BM * BK + w_lds;
+        uint8_t* bs = Bs + buf * BN * BK + w_lds;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) load16_to_lds(ap + a_goff[i], as + i * RPI * BK);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) load16_to_lds(bp + b_goff[i], bs + i * RPI * BK);
+    };
+
+    acc_t acc[TN][TM];
+    v4f accf[FOLD ? TN : 1][FOLD ? TM : 1];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b) acc[a][b] = acc_zero;
+    if constexpr (FOLD) {
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                const int m = m_base + b * 16, n = n_base + a * 16;
-                if (m >= p.M) continue;
-                acc_t t = acc[a][b];
-                if constexpr (B4) { t[0] >>= 4; t[1] >>= 4; t[2] >>= 4; t[3] >>= 4; }
-                acc_e* dst = static_cast<acc_e*>(p.C) + c_off + (int64_t)m * p.ldc + n;
-                if (p.vec_store && n + 3 < p.N) {
-                    *reinterpret_cast<acc_t*>(dst) = t;
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v)
-                        if (n + v < p.N) dst[v] = t[v];
-                }
-            }
-        return;
+            for (int b = 0; b < TM; ++b) accf[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
     }
 
-    float rx[TM];
-    if constexpr (!FOLD) range_rx(0, rx);
-    const bool is16 = p.out_dtype != SEGQ_F32;
-    const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
-    if (via_lds) {
-        // every wave transposes 16 rows at a time through its own patch of LDS
-        constexpr int RS = WN * 2 + 16;  // row stride in bytes; the 16 spreads rows over the banks
-        __syncthreads();                 // the operand tiles are dead from here on
-        uint8_t* patch = smem + wave * 16 * RS;
-        const int rd_row = lane / (WN / 8), rd_col = lane % (WN / 8);
-        constexpr int ROWS_PER_RD = 64 / (WN / 8);
-        float rwv[TN][4], bvv[TN][4];
+    const int f_sw = swz(lrow);
+    const int a_frag = (wm * WM + lrow) * BK;
+    const int b_frag = (wn * WN + lrow) * BK;
+    frag_t fa[2][TM], fb[2][TN];
+
+    // K half h of the tile in buffer buf -> fragment slot h
+    auto frags = [&](int buf, int h) {
+        const uint8_t* as = As + buf * BM * BK + a_frag;
+        const uint8_t* bs = Bs + buf * BN * BK + b_frag;
+        const int off = ((h * 4 + lgrp) ^ f_sw) << 4;
 #pragma unroll
-        for (int a = 0; a < TN; ++a) {
-            if constexpr (!FOLD) range_rw(0, a, rwv[a]);
+        for (int t = 0; t < TM; ++t) fa[h][t] = *reinterpret_cast<const v4i*>(as + t * 16 * BK + off);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
-        }
+        for (int t = 0; t < TN; ++t) fb[h][t] = *reinterpret_cast<const v4i*>(bs + t * 16 * BK + off);
+    };
+    auto mfmas = [&](int h) {
 #pragma unroll
-        for (int b = 0; b < TM; ++b) {
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[h][a], fa[h][b], acc[a][b], 0, 0, 0);
+    };
+
+    const int m_base = m0 + wm * WM + lrow;
+    const int n_base = n0 + wn * WN + 4 * lgrp;
+    auto fold = [&](int r) {
+        if constexpr (FOLD) {
+            const float* sx = p.r[r].sx + z * p.bsSx;
+            const float* sw = p.r[r].sw + z * p.bsSw;
+            const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs;
+            float rx[TM];
+#pragma unroll
+            for (int b = 0; b < TM; ++b) rx[b] = __builtin_amdgcn_rcpf(sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs]);
 #pragma unroll
             for (int a = 0; a < TN; ++a) {
-                uint32_t h[4];
+                float rw[4];
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float o = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
-                    h[v] = (p.out_dtype == SEGQ_BF16) ? f32_to_bf16_bits(o) : f32_to_f16_bits(o);
+                for (int v = 0; v < 4; ++v) rw[v] = __builtin_amdgcn_rcpf(sw[(int64_t)min(n_base + a * 16 + v, p.N - 1) * cs]);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) accf[a][b][v] += (float)acc[a][b][v] * rx[b] * rw[v];
+                    acc[a][b] = acc_zero;
                 }
-                *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
-                    make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
             }
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int j = 0; j < 16 / ROWS_PER_RD; ++j) {
-                const int row = j * ROWS_PER_RD + rd_row;
-                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + rd_col * 16);
-                const int m = m0 + wm * WM + b * 16 + row;
-                if (m < p.M)
-                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + rd_col * 8) = v;
-            }
-            __builtin_amdgcn_wave_barrier();
         }
-        return;
-    }
-#pragma unroll
-    for (int a = 0; a < TN; ++a) {
-        float rw[4];
-        if constexpr (!FOLD) range_rw(0, a, rw);
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (p.bias) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) bv[v] = load_bias(p.bias, p.bias_dtype, min(n_base + a * 16 + v, p.N - 1));
+    };
+
+    // (range, k) of the tile that is loaded two steps ahead of the one being multiplied
+    int lr = 0, lk = p.r[0].k0;
+    auto advance = [&](int& r, int& k) {
+        k += BK;
+        if (k >= p.r[r].k1) {
+            ++r;
+            k = (r < p.nr) ? p.r[r].k0 : 0;
         }
+    };
+    int steps = 0;
+    for (int i = 0; i < p.nr; ++i) steps += (p.r[i].k1 - p.r[i].k0) / BK;
+
+    // prologue: tiles 0 .. NS-1 on their way into buffers 0 .. NS-1; wait for tile 0
+    int issued = 0;
 #pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const int m = m_base + b * 16, n = n_base + a * 16;
-            if (m >= p.M || n >= p.N) continue;
-            float o[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
-                else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
-            }
-            const int64_t e = c_off + (int64_t)m * p.ldc + n;
-            const bool vec = p.vec_store && (n + 3 < p.N);
-            if (p.out_dtype == SEGQ_F32) store4<SEGQ_F32>(p.C, e, o, vec, p.N - n);
-            else if (p.out_dtype == SEGQ_BF16) store4<SEGQ_BF16>(p.C, e, o, vec, p.N - n);
-            else store4<SEGQ_F16>(p.C, e, o, vec, p.N - n);
+    for (int t = 0; t < NS; ++t) {
+        if (t < steps) {
+            dma(lr, lk, t);
+            advance(lr, lk);
+            ++issued;
         }
     }
+    if (issued == NS) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * (A_IT + B_IT)));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+    __syncthreads();
+    frags(0, 0);
+
+    int cr = 0, ck = p.r[0].k0;  // the tile being multiplied
+    int buf = 0;                  // its buffer, s % NS
+    for (int s = 0; s < steps; ++s) {
+        const bool last = s + 1 == steps;
+        const bool range_done = ck + BK >= p.r[cr].k1;
+        const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
+        frags(buf, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
+        // flight) and this wave's reads of tile s must be done, before anyone reads
+        // tile s+1 or overwrites the buffer of tile s.
+        if (s + NS - 1 < steps) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * (A_IT + B_IT)));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        __syncthreads();
+        if (s + NS < steps) {  // tile s+NS goes where tile s was: both its halves are in registers
+            dma(lr, lk, buf);
+            advance(lr, lk);
+        }
+        if (!last) frags(nbuf, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (FOLD && range_done) fold(cr);
+        advance(cr, ck);
+        buf = nbuf;
+    }
+    wide_epilogue<BM, BN, WGM, WGN, FMT, false, FOLD>(p, acc, accf, smem, z, m0, n0, wave, lane);
 }
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
@@ -377,8 +608,41 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 }
 
 // wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS>
+int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
+    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS>;
+    constexpr int lds = NS * (BM + BN) * BK;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", lds);
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    hipLaunchKernelGGL(kern, grid, dim3(WGM * WGN * 64), lds, st, p);
+    return check_launch("segq_gemm");
+}
+
 template <int FMT, bool B4>
 int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st) {
+    if constexpr (FMT == GEMM_I8 && !B4) {
+        if (!asel) {  // plain int8 operands: the software-pipelined kernel
+            if (!fold) {
+                switch (wcfg) {
+                    case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2>(p, batch, st);
+                    case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
+                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, false, 2>(p, batch, st);
+                }
+            } else {
+                switch (wcfg) {
+                    case 0: case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2>(p, batch, st);
+                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, true, 2>(p, batch, st);
+                }
+            }
+        }
+    }
 #define SEGQ_WIDE(BM_, BN_, WGM_, WGN_, FOLD_)                                                          \
     return asel ? launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, true>(p, batch, st)       \
                 : launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, false>(p, batch, st)
