@@ -165,16 +165,6 @@ __global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) 
 }
 
 // ---- dynamic per-row scales ------------------------------------------------
-__device__ __forceinline__ float block_max(float v, float* red) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    const int w = threadIdx.x >> 6;
-    __syncthreads();  // red may still be read from the previous reduction
-    if ((threadIdx.x & 63) == 0) red[w] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-}
-
 template <int FMT>
 __device__ __forceinline__ float qmax_pos() {
     return FMT == SEGQ_CODE_I8 ? 127.0f : (FMT == SEGQ_CODE_I4 ? 7.0f : 448.0f);
@@ -184,48 +174,115 @@ __device__ __forceinline__ float qmax_neg() {
     return FMT == SEGQ_CODE_I8 ? 128.0f : (FMT == SEGQ_CODE_I4 ? 8.0f : 448.0f);
 }
 
-// One block per row.  Up to CACHE runs per thread stay in registers between the
-// reduction and the encode; longer rows are read again (they hit in L2).
-template <int DT, int FMT>
+template <int DT>
+struct RawRun {  // 16 consecutive elements as they sit in memory
+    uint4 q[DT == SEGQ_F32 ? 4 : 2];
+};
+
+template <int DT>
+__device__ __forceinline__ void load_raw(const void* p, RawRun<DT>& r) {
+    const uint4* q = reinterpret_cast<const uint4*>(p);
+#pragma unroll
+    for (int i = 0; i < (DT == SEGQ_F32 ? 4 : 2); ++i) r.q[i] = q[i];
+}
+
+template <int DT>
+__device__ __forceinline__ void raw_to_f32(const RawRun<DT>& r, float (&v)[16]) {
+    if constexpr (DT == SEGQ_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[4 * i + 0] = __uint_as_float(r.q[i].x); v[4 * i + 1] = __uint_as_float(r.q[i].y);
+            v[4 * i + 2] = __uint_as_float(r.q[i].z); v[4 * i + 3] = __uint_as_float(r.q[i].w);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t w[4] = {r.q[i].x, r.q[i].y, r.q[i].z, r.q[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (DT == SEGQ_BF16) {
+                    v[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
+                    v[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                } else {
+                    v[8 * i + 2 * j + 0] = f16_bits_to_f32(w[j] & 0xffffu);
+                    v[8 * i + 2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+                }
+            }
+        }
+    }
+}
+
+// Running maxima of the positive and of the negative side (strict masks x > 0 and
+// x < 0, segquant/quantizers/quantizer.py:172-189; NaN is ignored).  Without
+// DualScale only their maximum matters, which is one max of |x| per element.
+template <bool DUAL>
+__device__ __forceinline__ void track_amax(const float (&v)[16], float& amax_p, float& amax_n) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        if constexpr (DUAL) {
+            amax_p = fmaxf(amax_p, v[j]);    // starts at 0, so negatives never win
+            amax_n = fmaxf(amax_n, -v[j]);
+        } else {
+            amax_p = fmaxf(amax_p, fabsf(v[j]));
+        }
+    }
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// One workgroup per row, for rows longer than a wave can hold.  All loads of
+// the row are issued before anything is computed; up to CACHE runs per thread
+// stay in registers in packed form between the reduction and the encode, longer
+// rows are read again (they hit in L2).
+template <int DT, int FMT, bool DUAL>
 __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p) {
     constexpr int CACHE = 4;
-    __shared__ float red_a[4];
-    __shared__ float red_b[4];
+    __shared__ float red[2][4];
     const int64_t row = blockIdx.x;
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
     const uint8_t* xrow = static_cast<const uint8_t*>(p.x) + row * p.ldx * esz;
     const float eps = 5.9604644775390625e-08f;  // 2^-24
-    const bool two = p.dual && p.codes_neg != nullptr;
+    const bool two = DUAL && p.codes_neg != nullptr;
     for (int ks = 0; ks < p.n_kseg; ++ks) {
         const int c0 = p.kb[ks] >> 4, c1 = p.kb[ks + 1] >> 4;
-        const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
-        float cache[CACHE][16];
+        const bool dual = DUAL && ((p.dual_mask >> ks) & 1u);
+        RawRun<DT> raw[CACHE];
+#pragma unroll
+        for (int i = 0; i < CACHE; ++i) {
+            const int c = c0 + threadIdx.x + i * 256;
+            if (c < c1) load_raw<DT>(xrow + (size_t)c * 16 * esz, raw[i]);
+        }
         float amax_p = 0.0f, amax_n = 0.0f;
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
             const int c = c0 + threadIdx.x + i * 256;
             if (c < c1) {
-                load16<DT>(xrow + (size_t)c * 16 * esz, cache[i]);
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const float a = cache[i][j];
-                    // strict masks: x > 0 and x < 0 (quantizer.py:172-189); NaN is ignored
-                    amax_p = fmaxf(amax_p, a > 0.0f ? a : 0.0f);
-                    amax_n = fmaxf(amax_n, a < 0.0f ? -a : 0.0f);
-                }
+                float v[16];
+                raw_to_f32<DT>(raw[i], v);
+                track_amax<DUAL>(v, amax_p, amax_n);
             }
         }
         for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
-            float t[16];
-            load16<DT>(xrow + (size_t)c * 16 * esz, t);
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                amax_p = fmaxf(amax_p, t[j] > 0.0f ? t[j] : 0.0f);
-                amax_n = fmaxf(amax_n, t[j] < 0.0f ? -t[j] : 0.0f);
-            }
+            RawRun<DT> t;
+            float v[16];
+            load_raw<DT>(xrow + (size_t)c * 16 * esz, t);
+            raw_to_f32<DT>(t, v);
+            track_amax<DUAL>(v, amax_p, amax_n);
         }
-        amax_p = block_max(amax_p, red_a);
-        amax_n = block_max(amax_n, red_b);
+        amax_p = wave_max(amax_p);
+        if constexpr (DUAL) amax_n = wave_max(amax_n);
+        __syncthreads();  // red may still be read from the previous column segment
+        if ((threadIdx.x & 63) == 0) {
+            red[0][threadIdx.x >> 6] = amax_p;
+            red[1][threadIdx.x >> 6] = amax_n;
+        }
+        __syncthreads();
+        amax_p = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+        amax_n = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
         float s_pos, s_neg;
         if (dual) {
             s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
@@ -236,17 +293,81 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
         const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
         if (threadIdx.x == 0) {
             p.scale[si] = s_pos;
-            if (p.dual) p.scale_neg[si] = s_neg;
+            if (DUAL) p.scale_neg[si] = s_neg;
         }
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
             const int c = c0 + threadIdx.x + i * 256;
-            if (c < c1) encode16<FMT>(p, row, (int64_t)c << 4, cache[i], s_pos, s_neg, two);
+            if (c < c1) {
+                float v[16];
+                raw_to_f32<DT>(raw[i], v);
+                encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
+            }
         }
         for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
-            float t[16];
-            load16<DT>(xrow + (size_t)c * 16 * esz, t);
-            encode16<FMT>(p, row, (int64_t)c << 4, t, s_pos, s_neg, two);
+            RawRun<DT> t;
+            float v[16];
+            load_raw<DT>(xrow + (size_t)c * 16 * esz, t);
+            raw_to_f32<DT>(t, v);
+            encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
+        }
+    }
+}
+
+// ---- dynamic per-row scales, one WAVE per row --------------------------------
+// For rows of up to 64 * CPL runs: the whole row is in flight at once, the
+// maximum is reduced with cross-lane shuffles only, and four rows share a
+// workgroup without ever synchronising.
+template <int DT, int FMT, int CPL, bool DUAL>
+__global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= p.rows) return;
+    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+    const uint8_t* xrow = static_cast<const uint8_t*>(p.x) + row * p.ldx * esz;
+    const float eps = 5.9604644775390625e-08f;  // 2^-24
+    const bool two = DUAL && p.codes_neg != nullptr;
+    for (int ks = 0; ks < p.n_kseg; ++ks) {
+        const int c0 = p.kb[ks] >> 4, c1 = p.kb[ks + 1] >> 4;
+        const bool dual = DUAL && ((p.dual_mask >> ks) & 1u);
+        RawRun<DT> raw[CPL];
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            const int c = c0 + lane + i * 64;
+            if (c < c1) load_raw<DT>(xrow + (size_t)c * 16 * esz, raw[i]);
+        }
+        float amax_p = 0.0f, amax_n = 0.0f;
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            const int c = c0 + lane + i * 64;
+            if (c < c1) {
+                float v[16];
+                raw_to_f32<DT>(raw[i], v);
+                track_amax<DUAL>(v, amax_p, amax_n);
+            }
+        }
+        amax_p = wave_max(amax_p);
+        if constexpr (DUAL) amax_n = wave_max(amax_n);
+        float s_pos, s_neg;
+        if (dual) {
+            s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
+            s_neg = qmax_neg<FMT>() / fmaxf(amax_n, eps);
+        } else {
+            s_pos = s_neg = qmax_pos<FMT>() / fmaxf(fmaxf(amax_p, amax_n), eps);
+        }
+        const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
+        if (lane == 0) {
+            p.scale[si] = s_pos;
+            if (DUAL) p.scale_neg[si] = s_neg;
+        }
+#pragma unroll
+        for (int i = 0; i < CPL; ++i) {
+            const int c = c0 + lane + i * 64;
+            if (c < c1) {
+                float v[16];
+                raw_to_f32<DT>(raw[i], v);
+                encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
+            }
         }
     }
 }
@@ -276,7 +397,16 @@ __global__ void __launch_bounds__(256) fake_e4m3_kernel(const void* x, void* out
 template <int DT, int FMT>
 static int launch_quant(const QuantParams& p, hipStream_t st) {
     if (p.dynamic) {
-        hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT>), dim3((unsigned)p.rows), dim3(256), 0, st, p);
+        int longest = 0;  // runs of 16 in the longest column segment
+        for (int i = 0; i < p.n_kseg; ++i) longest = longest > (p.kb[i + 1] - p.kb[i]) / 16 ? longest : (p.kb[i + 1] - p.kb[i]) / 16;
+        const dim3 wgrid((unsigned)((p.rows + 3) / 4)), bgrid((unsigned)p.rows);
+        if (longest <= 64 * 4) {
+            if (p.dual) hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, true>), wgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, false>), wgrid, dim3(256), 0, st, p);
+        } else {
+            if (p.dual) hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, true>), bgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, false>), bgrid, dim3(256), 0, st, p);
+        }
     } else {
         const int64_t runs = p.rows * (p.cols >> 4);
         hipLaunchKernelGGL((quant_static_kernel<DT, FMT>), dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, st, p);
