@@ -71,6 +71,8 @@ def main():
     ap.add_argument("--config", type=int, default=3, help="benchmark configuration 1..5 (default: FLUX int8, M=4608)")
     ap.add_argument("--cpu-rows", type=int, default=512, help="tokens per linear in the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -103,6 +105,12 @@ def main():
         for layer, x in zip(layers, xs):
             layer(x)
 
+    if args.calib_copy:
+        src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
