@@ -418,15 +418,30 @@ def int_qrange(bits: int):
     return -(2 ** (bits - 1)), 2 ** (bits - 1) - 1  # quantizer.py:151-152
 
 
+def _scalar_over_tensor(limit, amax) -> np.ndarray:
+    """``limit / tensor`` as torch evaluates it for a python scalar on the left:
+    ``tensor.reciprocal() * limit``, two fp32 roundings (torch/_tensor.py,
+    ``__rtruediv__``).  This is what the reference's per-axis formulas compute."""
+    clamped = np.maximum(_f32(amax), np.float32(EPS))
+    return ((np.float32(1.0) / clamped) * np.float32(limit)).astype(np.float32)
+
+
+def row_scale_div(amax, limit) -> np.ndarray:
+    """``limit / max(amax, eps)`` as ONE correctly rounded fp32 division: the
+    definition the quantise kernel uses for dynamic per-row scales (which the
+    reference has no working counterpart of, optimum/optimizer.py:96-100)."""
+    return (np.float32(limit) / np.maximum(_f32(amax), np.float32(EPS))).astype(np.float32)
+
+
 def int_scale(amax, bits: int = 8):
     """Symmetric per-tensor: ``qmax/amax`` if amax > eps else 1.0 (python float
     arithmetic, quantizer.py:206-210).  Array input: ``qmax / clamp(amax, eps)``
-    in fp32 (quantizer.py:211-219)."""
+    evaluated by torch in fp32 (quantizer.py:211-219)."""
     _, qmax = int_qrange(bits)
     if np.ndim(amax) == 0:
         amax = float(amax)
         return qmax / amax if amax > EPS else 1.0
-    return (np.float32(qmax) / np.maximum(_f32(amax), np.float32(EPS))).astype(np.float32)
+    return _scalar_over_tensor(qmax, amax)
 
 
 def int_dual_scales(pos_amax, neg_amax, bits: int = 8):
@@ -437,9 +452,8 @@ def int_dual_scales(pos_amax, neg_amax, bits: int = 8):
         neg = qmin / (-neg_amax) if neg_amax > EPS else 1.0
         pos = qmax / pos_amax if pos_amax > EPS else 1.0
         return pos, neg
-    neg = np.float32(qmin) / (-np.maximum(_f32(neg_amax), np.float32(EPS)))
-    pos = np.float32(qmax) / np.maximum(_f32(pos_amax), np.float32(EPS))
-    return pos.astype(np.float32), neg.astype(np.float32)
+    # qmin / (-clamp(neg_amax)): the same reciprocal-times-scalar, signs cancel exactly
+    return _scalar_over_tensor(qmax, pos_amax), _scalar_over_tensor(-qmin, neg_amax)
 
 
 def fp8_scale(amax):
@@ -447,7 +461,7 @@ def fp8_scale(amax):
     if np.ndim(amax) == 0:
         amax = float(amax)
         return 448.0 / amax if amax > EPS else 1.0
-    return (np.float32(448.0) / np.maximum(_f32(amax), np.float32(EPS))).astype(np.float32)
+    return _scalar_over_tensor(448.0, amax)
 
 
 def fp8_dual_scales(pos_amax, neg_amax):

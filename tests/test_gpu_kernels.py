@@ -143,15 +143,17 @@ def test_quantize_dynamic_per_row(ops, fmt, dual):
     c = ops.quantize(x, fmt, s, sn, row_stride=1, dual=dual, dynamic=True)
     xn = _np(x)
     bits = 4 if fmt == O.FMT_INT4 else 8
+    lim_p = {O.FMT_INT8: 127.0, O.FMT_INT4: 7.0, O.FMT_E4M3: 448.0}[fmt]
+    lim_n = {O.FMT_INT8: 128.0, O.FMT_INT4: 8.0, O.FMT_E4M3: 448.0}[fmt]
     if dual:
         pa, na = O.dual_amax(xn, axis=-1)
-        ws, wn = O.fp8_dual_scales(pa, na) if fmt == O.FMT_E4M3 else O.int_dual_scales(pa, na, bits)
+        ws, wn = O.row_scale_div(pa, lim_p), O.row_scale_div(na, lim_n)
         assert np.array_equal(s.cpu().numpy(), ws) and np.array_equal(sn.cpu().numpy(), wn)
         wp, wq = O.quantize_act_dual(xn[None], ws, wn, fmt)
         want = O.merge_dual_codes(wp, wq, xn[None])[0]
     else:
         amax = np.abs(xn).max(axis=-1)
-        ws = O.fp8_scale(amax) if fmt == O.FMT_E4M3 else O.int_scale(amax, bits)
+        ws = O.row_scale_div(amax, lim_p)
         assert np.array_equal(s.cpu().numpy(), ws)
         want = O.quantize_act(xn[None], ws, fmt)[0]
     assert np.array_equal(_codes_np(c, fmt), want)

@@ -60,11 +60,14 @@ def oracle_layer_output(layer, spec, x_np, out_dtype):
         xs = x_np[:, k0:k1]
         cal = opt.input_calibrators[s if spec.seg_mode == "input" else 0]
         dual = opt.dual_segments[s if spec.seg_mode == "input" else 0]
-        if spec.dynamic:
+        if spec.dynamic:  # the kernel's own definition: one fp32 division per row
+            lim_p = {O.FMT_INT8: 127.0, O.FMT_INT4: 7.0, O.FMT_E4M3: 448.0}[fa]
+            lim_n = {O.FMT_INT8: 128.0, O.FMT_INT4: 8.0, O.FMT_E4M3: 448.0}[fa]
             if dual:
-                ps, ns = dualf(*O.dual_amax(xs, axis=-1))
+                pa, na = O.dual_amax(xs, axis=-1)
+                ps, ns = O.row_scale_div(pa, lim_p), O.row_scale_div(na, lim_n)
             else:
-                ps = single(np.abs(xs).max(axis=-1))
+                ps = O.row_scale_div(np.abs(xs).max(axis=-1), lim_p)
         else:
             if dual:
                 ps, ns = (np.float32(_np32(torch.as_tensor(t))) for t in (cal.pos_scale, cal.neg_scale))

@@ -1,0 +1,332 @@
+"""CPU tests: the C-ABI library loads and exports what include/segq.h declares,
+and the host-side mirror (quantisers, calibrators, optimiser, SegmentLinear,
+quantize()) computes the reference's fake-quant arithmetic, checked against the
+numpy oracle.  No GPU compute happens here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fake_path_torch as F
+from oracle import segq_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------ the C ABI
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "segq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(segq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from segquant_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared_symbols()
+    assert set(declared) == set(_lib.EXPORTS), (declared, _lib.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.segq_version.restype = ctypes.c_int
+    assert lib.segq_version() >= 100
+    lib.segq_gemm_tile_count.restype = ctypes.c_int
+    assert lib.segq_gemm_tile_count() >= 5
+
+
+def test_struct_layouts_match_the_header():
+    """ctypes mirrors must have the size the C compiler gives the header's structs."""
+    import subprocess
+    import tempfile
+    from segquant_amd import _lib
+    src = ('#include "segq.h"\n#include <stdio.h>\nint main(){printf("%zu %zu %zu\\n",'
+           'sizeof(segq_quant_desc),sizeof(segq_krange),sizeof(segq_gemm_desc));return 0;}\n')
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "s.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "s")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        sizes = [int(t) for t in subprocess.run([exe], capture_output=True, text=True, check=True).stdout.split()]
+    assert sizes == [ctypes.sizeof(_lib.QuantDesc), ctypes.sizeof(_lib.KRange), ctypes.sizeof(_lib.GemmDesc)]
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    from segquant_amd import _lib
+    lib = _lib.lib()
+    d = _lib.GemmDesc()
+    d.m, d.n, d.batch = 4, 4, 1
+    assert lib.segq_gemm(ctypes.byref(d), None) == 1  # SEGQ_ERR_ARG: null pointers
+    assert b"null" in lib.segq_last_error()
+    q = _lib.QuantDesc()
+    q.rows, q.cols = 2, 24  # cols not a multiple of 16
+    q.x = q.codes = q.scale = 16
+    assert lib.segq_quantize(ctypes.byref(q), None) == 1
+    assert b"multiple of 16" in lib.segq_last_error()
+    with pytest.raises(RuntimeError):
+        _lib.check(1)
+
+
+# ------------------------------------------------------------------ registry / loaders
+def test_ext_dict_has_the_reference_shape():
+    from segquant_amd.layers import ext_dict
+    from segquant_amd.utils import extension as E
+    assert set(ext_dict) == set(E.supported_type)
+    for entry in ext_dict.values():
+        assert set(entry) == {"gemm_scaled_fn", "gemm_dual_scaled_fn"}
+    if not torch.cuda.is_available():
+        assert all(v is None for e in ext_dict.values() for v in e.values())
+        ext, prefixes = E.load_real_quant_int8_ext(required=False)
+        assert ext is None and prefixes == ("Wint8Aint8",)
+        with pytest.raises(RuntimeError):
+            E.load_real_quant_int8_ext(required=True)
+
+
+def test_real_quant_without_gpu_raises_instead_of_falling_back():
+    if torch.cuda.is_available():
+        pytest.skip("needs a machine without a GPU")
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    with pytest.raises(RuntimeError):
+        SegmentLinear(32, 16, input_quant_type="int8", weight_quant_type="int8",
+                      input_quant_args={"real_quant": True}, weight_quant_args={"real_quant": True}, device="cpu")
+
+
+def test_fake_e4m3fy_cpu_matches_oracle():
+    from segquant_amd.utils.extension import load_fake_quant_fp8_ext
+    x = torch.randn(5000) * 100
+    x[:4] = torch.tensor([0.0, 1e9, -1e9, 2.0 ** -10])
+    got = load_fake_quant_fp8_ext().fake_e4m3fy(x).numpy()
+    assert np.array_equal(got, O.e4m3_roundtrip(x.numpy()))
+
+
+# ------------------------------------------------------------------ quantisers
+@pytest.mark.parametrize("bits", [8, 4])
+def test_int_quantizer_scales_and_fake_quant(bits):
+    from segquant_amd.quantizers.quantizer import IntQuantizer
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(6, 32, generator=g) * 3
+    q = IntQuantizer(num_bits=bits)
+    q.calibrate(x)
+    q.calibrate(x * 0.5)  # running maximum keeps the larger one
+    assert q.scale == O.int_scale(float(x.abs().max()), bits)
+    assert np.array_equal(q.fake_quantize(x).numpy(), O.fake_quant_int(x.numpy(), np.float32(q.scale), bits))
+    qa = IntQuantizer(num_bits=bits, axis=-1)
+    qa.calibrate(x)
+    assert np.array_equal(qa.scale.numpy(), O.int_scale(x.abs().amax(-1).numpy(), bits))
+    qd = IntQuantizer(num_bits=bits, dual_scale=True)
+    qd.calibrate(x)
+    pos, neg = O.int_dual_scales(*O.dual_amax(x.numpy()), bits)
+    assert (qd.pos_scale, qd.neg_scale) == (pos, neg)
+    assert np.array_equal(qd.fake_quantize(x).numpy(),
+                          O.fake_quant_int_dual(x.numpy(), np.float32(pos), np.float32(neg), bits))
+    qz = IntQuantizer(num_bits=bits, dual_scale=True)
+    qz.calibrate(torch.zeros(4, 4))
+    assert (qz.pos_scale, qz.neg_scale) == (1.0, 1.0)
+
+
+def test_float_quantizer_scales_and_fake_quant():
+    from segquant_amd.quantizers.quantizer import FloatQuantizer, QuantizerRegistry
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(8, 48, generator=g)
+    x[0, 0] = 2.0 ** -26
+    q = QuantizerRegistry.create("fpe4m3")
+    assert isinstance(q, FloatQuantizer)
+    q.calibrate(x)
+    assert q.scale == O.fp8_scale(float(x.abs().max()))
+    assert np.array_equal(q.fake_quantize(x).numpy(), O.fake_quant_fp8(x.numpy(), np.float32(q.scale)))
+    qd = FloatQuantizer(dual_scale=True, axis=-1)
+    qd.calibrate(x)
+    pa, na = O.dual_amax(x.numpy(), axis=-1)
+    ps, ns = O.fp8_dual_scales(pa, na)
+    assert np.array_equal(qd.pos_scale.numpy(), ps) and np.array_equal(qd.neg_scale.numpy(), ns)
+    want = O.fake_quant_fp8_dual(x.numpy(), ps[:, None], ns[:, None])
+    assert np.array_equal(qd.fake_quantize(x).numpy(), want)
+    a = FloatQuantizer._simulate_fp(x * 10, q.fp_min, q.fp_max, 3).numpy()
+    assert np.array_equal(a, O.simulate_fp((x * 10).numpy(), O.E4M3_FP_MIN, 448.0, 3))
+
+
+def test_registry_names_follow_dtype_values():
+    from segquant_amd.config import DType
+    from segquant_amd.quantizers.quantizer import QuantizerRegistry
+    for d in DType:
+        assert QuantizerRegistry.get(d.value) is not None, d
+    assert QuantizerRegistry.create("int4").qmax == 7
+    with pytest.raises(ValueError):
+        QuantizerRegistry.create("nope")
+
+
+# ------------------------------------------------------------------ SegmentLinear, fake path
+def _make_layer(K, N, seg_mode, chunks, chunksizes=None, atype="int8", wtype="int8", axis=False, dual=False, seed=0):
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(N, K, generator=g) * 0.05
+    b = torch.randn(N, generator=g) * 0.01
+    layer = SegmentLinear(K, N, bias=True, seg_mode=seg_mode, chunks=chunks, chunksizes=chunksizes,
+                          custom_weight_tensor=w, custom_bias_tensor=b, input_quant_type=atype,
+                          weight_quant_type=wtype,
+                          input_quant_args={"real_quant": False, "dual_scale": dual, "axis": -1 if axis else None},
+                          weight_quant_args={"real_quant": False, "axis": 1 if axis else None}, device="cpu")
+    return layer, w, b
+
+
+@pytest.mark.parametrize("seg_mode,chunks", [("weight", 1), ("weight", 3), ("input", 2)])
+@pytest.mark.parametrize("axis", [False, True])
+@pytest.mark.parametrize("atype", ["int8", "fpe4m3"])
+def test_segment_linear_fake_path_equals_oracle(seg_mode, chunks, axis, atype):
+    M, K, N = 7, 64, 48
+    layer, w, b = _make_layer(K, N, seg_mode, chunks, atype=atype, wtype=atype, axis=axis)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g)
+    x_before = x.clone()
+    layer.calibrate(x)
+    layer.finish_calibrate()
+    y = layer(x).numpy()
+    assert torch.equal(x, x_before), "the fake path must not write into the caller's input"
+    # oracle: same segment views, per-segment scales by the closed forms
+    xs, ws = O.segment_views(x.numpy(), w.numpy(), seg_mode, chunks)
+    sc = (lambda a: O.fp8_scale(a)) if atype == "fpe4m3" else (lambda a: O.int_scale(a, 8))
+    fq = (lambda t, s: O.fake_quant_fp8(t, s)) if atype == "fpe4m3" else (lambda t, s: O.fake_quant_int(t, s, 8))
+    outs = []
+    for s in range(chunks):
+        xi = np.ascontiguousarray(xs[s])
+        wi = np.ascontiguousarray(ws[s]) if seg_mode == "weight" else w.numpy()
+        if axis:
+            sx = sc(np.abs(xi).max(-1))[:, None]
+            sw_full = sc(np.abs(wi).max(-1))[:, None]
+        else:
+            sx = np.float32(sc(float(np.abs(xi).max())))
+            sw_full = np.float32(sc(float(np.abs(wi).max())))
+        wq = fq(wi, sw_full)
+        if seg_mode == "input":
+            wq = wq[:, s * (K // chunks):(s + 1) * (K // chunks)]
+        outs.append(fq(xi, sx) @ wq.T)
+    want = O.recombine(np.stack(outs), seg_mode, bias=b.numpy())
+    assert np.abs(y - want).max() <= 2e-6 * np.abs(want).max()
+    # chunked output has the reference's (S, ..., n) layout
+    ch = layer(x, chunked=True)
+    assert ch.shape == (chunks, M, N // chunks if seg_mode == "weight" else N)
+
+
+def test_unequal_and_mixed_dual_segments_on_the_fake_path():
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    K, N, M = 96, 40, 9
+    g = torch.Generator().manual_seed(2)
+    w = torch.randn(N, K, generator=g) * 0.05
+    x = torch.randn(M, K, generator=g)
+    x[:, 32:] = torch.nn.functional.gelu(x[:, 32:])
+    layer = SegmentLinear(K, N, bias=False, seg_mode="input", chunks=2, chunksizes=[32, 64], custom_weight_tensor=w,
+                          input_quant_type="int8", weight_quant_type="int8",
+                          input_quant_args={"real_quant": False, "dual_scale": [False, True], "axis": None},
+                          weight_quant_args={"real_quant": False, "axis": None}, device="cpu")
+    assert layer.optimizer.dual_segments == [False, True] and layer.optimizer.dual_scale
+    layer.calibrate(x)
+    layer.finish_calibrate()
+    y = layer(x).numpy()
+    xn, wn = x.numpy(), w.numpy()
+    s0 = np.float32(O.int_scale(float(np.abs(xn[:, :32]).max())))
+    ps, ns = (np.float32(t) for t in O.int_dual_scales(*O.dual_amax(xn[:, 32:])))
+    sw = np.float32(O.int_scale(float(np.abs(wn).max())))
+    xf = np.concatenate([O.fake_quant_int(xn[:, :32], s0), O.fake_quant_int_dual(xn[:, 32:], ps, ns)], axis=1)
+    want = xf @ O.fake_quant_int(wn, sw).T
+    assert np.abs(y - want).max() <= 2e-6 * np.abs(want).max()
+    with pytest.raises(NotImplementedError):
+        layer(x, chunked=True)  # stacked per-segment outputs need equal sizes, as in the reference
+
+
+def test_constructor_checks_mirror_the_reference():
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    with pytest.raises(ValueError):
+        SegmentLinear(8, 8, seg_mode="rows", input_quant_type="int8", weight_quant_type="int8", device="cpu")
+    with pytest.raises(AssertionError):
+        SegmentLinear(8, 8, custom_weight_tensor=torch.zeros(4, 8), input_quant_type="int8",
+                      weight_quant_type="int8", device="cpu")
+    with pytest.raises(ValueError):
+        SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8",
+                      weight_quant_args={"dual_scale": True}, device="cpu")
+    with pytest.raises(NotImplementedError):
+        SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8", opt_type="smooth", device="cpu")
+
+
+def test_quantize_replaces_linears_and_keeps_outputs_close():
+    from segquant_amd.config import Calibrate, DType, Optimum
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    from segquant_amd.torch.quantization import quantize
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(32, 32)
+            self.blocks = torch.nn.ModuleList([torch.nn.Linear(64, 48), torch.nn.Linear(48, 16)])
+            self.skip = torch.nn.Linear(16, 16)
+
+        def forward(self, x, e):
+            h = torch.cat([self.a(x), e], dim=1)
+            return self.skip(self.blocks[1](torch.nn.functional.silu(self.blocks[0](h))))
+
+    torch.manual_seed(0)
+    net = Net()
+    g = torch.Generator().manual_seed(42)
+    loader = [((torch.rand(3, 32, generator=g), torch.rand(3, 32, generator=g)),) for _ in range(5)]
+    cfg = {"default": {"enable": True, "seglinear": True, "search_patterns": [], "real_quant": False,
+                       "opt": {"type": Optimum.DEFAULT}, "calib": {"type": Calibrate.AMAX},
+                       "input_quant": {"type": DType.INT8, "axis": None},
+                       "weight_quant": {"type": DType.INT8, "axis": None}},
+           "skip": {"enable": False}}
+    x, e = torch.rand(3, 32, generator=g), torch.rand(3, 32, generator=g)
+    ref = net(x, e)
+    import copy
+    qnet = quantize(copy.deepcopy(net), loader, cfg, seg_configs={"blocks.0": {"seg_mode": "input", "chunks": 2}},
+                    dual_scale_linears={"blocks.1"})
+    assert isinstance(qnet.a, SegmentLinear) and isinstance(qnet.blocks[0], SegmentLinear)
+    assert isinstance(qnet.skip, torch.nn.Linear)  # disabled by pattern
+    assert qnet.blocks[0].seg_mode == "input" and qnet.blocks[0].chunks == 2
+    assert qnet.blocks[1].optimizer.dual_scale and not qnet.a.optimizer.dual_scale
+    out = qnet(x, e)
+    assert ((out - ref).norm() / ref.norm()).item() < 0.05
+    off = copy.deepcopy(cfg)
+    off["default"]["enable"] = False
+    same = quantize(copy.deepcopy(net), loader, off)
+    assert isinstance(same.a, torch.nn.Linear)
+
+
+# ------------------------------------------------------------------ workloads and the CPU baseline
+def test_workloads_are_deterministic_and_shaped_like_the_configs():
+    from segquant_amd import workloads as W
+    shapes = {1: [(256, 1536, 9216)], 2: [(4096, 1536, 6144), (4096, 6144, 1536)],
+              3: [(4608, 3072, 9216), (4608, 3072, 12288), (4608, 12288, 3072)],
+              4: [(8192, 1280, 10240), (8192, 5120, 1280), (2048, 1280, 10240)]}
+    for c, want in shapes.items():
+        assert [(s.M, s.K, s.N) for s in W.config_linears(c)] == want
+    c5 = W.config_linears(5)
+    assert sorted({s.M for s in c5}) == [1024, 4608, 9216] and all(s.chunksizes == [3072, 12288] for s in c5)
+    sp = W.config_linears(3, M=8)[0]
+    a, b = W.make_input(sp), W.make_input(sp)
+    assert torch.equal(a, b) and a.shape == (8, 3072)
+    assert not torch.equal(W.make_weight(sp), W.make_weight(W.config_linears(3, M=8)[1])[:9216])
+
+
+def test_torch_fake_path_equals_numpy_oracle():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(12, 96, generator=g)
+    x[:, 32:] = torch.nn.functional.gelu(x[:, 32:])
+    w = torch.randn(20, 96, generator=g) * 0.05
+    for fmt in ("int8", "fpe4m3"):
+        sw = F.scale_of(w.abs().amax(), fmt)
+        w_hat = F.fake_quant(w, fmt, sw)
+        y = F.fake_linear(x, w_hat, None, fmt, [0, 32, 96], [False, True], per_token=True).numpy()
+        xn = x.numpy()
+        sc, dsc = (O.fp8_scale, O.fp8_dual_scales) if fmt == "fpe4m3" else (O.int_scale, O.int_dual_scales)
+        s0 = sc(np.abs(xn[:, :32]).max(-1))[:, None]
+        pa, na = O.dual_amax(xn[:, 32:], axis=-1)
+        ps, ns = dsc(pa, na)
+        if fmt == "fpe4m3":
+            xf = np.concatenate([O.fake_quant_fp8(xn[:, :32], s0), O.fake_quant_fp8_dual(xn[:, 32:], ps[:, None], ns[:, None])], 1)
+            wf = O.fake_quant_fp8(w.numpy(), np.float32(sw))
+        else:
+            xf = np.concatenate([O.fake_quant_int(xn[:, :32], s0), O.fake_quant_int_dual(xn[:, 32:], ps[:, None], ns[:, None])], 1)
+            wf = O.fake_quant_int(w.numpy(), np.float32(sw))
+        want = xf @ wf.T
+        assert np.abs(y - want).max() <= 2e-6 * np.abs(want).max()

@@ -237,6 +237,13 @@ def test_scale_closed_forms():
     assert O.fp8_scale(7.0) == 64.0 and O.fp8_dual_scales(7.0, 14.0) == (64.0, 32.0)
     v = O.int_scale(np.float32([0.0, 1.0]))
     assert v[0] == np.float32(127.0) / np.float32(2.0 ** -24) and v[1] == 127.0
+    # per-axis scales follow torch's scalar / tensor = reciprocal * scalar
+    a = torch.rand(1000, generator=torch.Generator().manual_seed(3)) * 10 + 0.01
+    assert np.array_equal(O.int_scale(a.numpy()), (127 / a.clamp(min=O.EPS)).numpy())
+    assert np.array_equal(O.fp8_scale(a.numpy()), (448.0 / a.clamp(min=O.EPS)).numpy())
+    p_, n_ = O.int_dual_scales(a.numpy(), a.numpy())
+    assert np.array_equal(n_, (-128 / (-a.clamp(min=O.EPS))).numpy()) and np.array_equal(p_, O.int_scale(a.numpy()))
+    assert np.array_equal(O.row_scale_div(a.numpy(), 127.0), (torch.full_like(a, 127.0) / a).numpy())
     p, n = O.dual_amax(np.float32([[-3, 0, 2], [0, 0, 0]]), axis=-1)
     assert p.tolist() == [2, 0] and n.tolist() == [3, 0]
     assert O.dual_amax(np.float32([1, 2])) == (2.0, 0.0)
