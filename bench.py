@@ -19,6 +19,10 @@ if ROOT not in sys.path:
 
 PEAK_TOPS = {"int8": 5000.0, "fpe4m3": 5000.0}  # dense MFMA, TOP/s
 PEAK_HBM = 8000.0                               # GB/s
+# HBM-side bytes per GEMM launch (fetched + written), from the two rocprofv3 --pmc runs
+# summarised in profiles/gemm_pipe_int8_flux_m4608.md (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB,
+# factors from a 256 MiB copy).  Counters cannot be read from inside this process.
+MEASURED_TRAFFIC_BYTES = {3: 401.1e6}
 
 
 def cpu_baseline(specs, rows, repeats=3):
@@ -124,7 +128,7 @@ def main():
     total_ops = sum(sp.ops for sp in specs)
     value = total_ops * args.steps / wall / 1e12
 
-    g_t = g_ops = g_exec = q_t = q_bytes = 0.0
+    g_t = g_ops = g_exec = g_bytes = q_t = q_bytes = 0.0
     n_g = n_q = 0
     for kind, e0, e1, info in log:
         ms = e0.elapsed_time(e1)
@@ -132,6 +136,8 @@ def main():
             g_t += ms * 1e-3
             g_ops += 2.0 * info["m"] * info["n"] * info["k_alg"] * info["batch"]
             g_exec += 2.0 * info["m"] * info["n"] * info["k_exec"] * info["batch"]
+            g_bytes += info["batch"] * (info["m"] * info["k_alg"] + info["n"] * info["k_alg"] * (0.5 if info["b_fmt"] == "int4" else 1.0)
+                                        + 2.0 * info["m"] * info["n"])
             n_g += 1
         else:
             q_t += ms * 1e-3
@@ -150,8 +156,9 @@ def main():
                    "step": "activation quantize + segmented GEMM with fused dequant+bias, per linear",
                    "input_dtype": str(specs[0].x_dtype).replace("torch.", ""), "output_dtype": str(specs[0].x_dtype).replace("torch.", "")},
         "roofline": {"bound": "mfma", "kernel": "segq::gemm_kernel", "achieved": round(g_tops, 2), "peak": peak,
-                     "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
                      "launches": n_g, "avg_launch_us": round(g_t / max(n_g, 1) * 1e6, 2),
+                     "algorithmic_bytes_per_launch": round(g_bytes / max(n_g, 1)),
                      "executed_tops": round(g_exec / g_t / 1e12, 2)},
         "quantize": {"bound": "hbm", "kernel": "segq::quant_*_kernel", "achieved": round(q_gbs, 1), "peak": PEAK_HBM,
                      "unit": "GB/s", "frac": round(q_gbs / PEAK_HBM, 4), "launches": n_q,
