@@ -78,7 +78,8 @@ const char* segq_last_error(void);
  * says whether column segment i is dual; other segments use scale[] for both
  * signs.  With codes_neg == NULL one merged code tensor is written (the code of
  * the branch that was taken); with codes_neg != NULL the reference's two
- * tensors are written, Xp to codes and Xn to codes_neg.
+ * tensors are written, Xp to codes and Xn to codes_neg (column segments that are
+ * not dual write their one code to codes and leave codes_neg untouched).
  *
  * dynamic != 0: scale[] (and scale_neg[]) are OUTPUTS.  The kernel takes the
  * absolute maximum of every (row, column segment), writes

@@ -161,7 +161,8 @@ __global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) 
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
     float x[16];
     load16<DT>(static_cast<const uint8_t*>(p.x) + (row * p.ldx + col) * esz, x);
-    encode16<FMT>(p, row, col, x, s_pos, s_neg, p.dual && p.codes_neg != nullptr);
+    // the second tensor exists only for DualScale column segments
+    encode16<FMT>(p, row, col, x, s_pos, s_neg, dual && p.codes_neg != nullptr);
 }
 
 // ---- dynamic per-row scales ------------------------------------------------
@@ -246,10 +247,10 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
     const uint8_t* xrow = static_cast<const uint8_t*>(p.x) + row * p.ldx * esz;
     const float eps = 5.9604644775390625e-08f;  // 2^-24
-    const bool two = DUAL && p.codes_neg != nullptr;
     for (int ks = 0; ks < p.n_kseg; ++ks) {
         const int c0 = p.kb[ks] >> 4, c1 = p.kb[ks + 1] >> 4;
         const bool dual = DUAL && ((p.dual_mask >> ks) & 1u);
+        const bool two = dual && p.codes_neg != nullptr;  // the second tensor exists only for DualScale segments
         RawRun<DT> raw[CACHE];
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
@@ -326,10 +327,10 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
     const uint8_t* xrow = static_cast<const uint8_t*>(p.x) + row * p.ldx * esz;
     const float eps = 5.9604644775390625e-08f;  // 2^-24
-    const bool two = DUAL && p.codes_neg != nullptr;
     for (int ks = 0; ks < p.n_kseg; ++ks) {
         const int c0 = p.kb[ks] >> 4, c1 = p.kb[ks + 1] >> 4;
         const bool dual = DUAL && ((p.dual_mask >> ks) & 1u);
+        const bool two = dual && p.codes_neg != nullptr;  // the second tensor exists only for DualScale segments
         RawRun<DT> raw[CPL];
 #pragma unroll
         for (int i = 0; i < CPL; ++i) {

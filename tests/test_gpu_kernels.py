@@ -127,6 +127,12 @@ def test_quantize_column_segments_with_partial_dual(ops):
     wp, wn = O.quantize_act_dual(xn[None, :, 48:], np.float32([20.0]), np.float32([40.0]), O.FMT_INT8)
     w1 = O.merge_dual_codes(wp, wn, xn[None, :, 48:])[0]
     assert np.array_equal(c.cpu().numpy(), np.concatenate([w0, w1], axis=1))
+    # two-tensor layout: the plain segment keeps its one code in the first tensor
+    xn_t = torch.full((M, K), 77, dtype=torch.int8, device=DEV)
+    xp_t, xn_t = ops.quantize(x, O.FMT_INT8, pos, neg, kseg_bounds=bounds, kseg_stride=1, dual=True,
+                              dual_kseg_mask=0b10, two_tensors=True, out_neg=xn_t)
+    assert np.array_equal(xp_t.cpu().numpy(), np.concatenate([w0, wp[0]], axis=1))
+    assert np.array_equal(xn_t.cpu().numpy()[:, 48:], wn[0]) and (xn_t.cpu().numpy()[:, :48] == 77).all()
 
 
 @pytest.mark.parametrize("fmt", FMTS)
