@@ -560,6 +560,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
     __syncthreads();
     frags(0, 0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop head must see F0 as landed on every path
 
     int cr = 0, ck = p.r[0].k0;  // the tile being multiplied
     int buf = 0;                  // its buffer, s % NS
@@ -585,6 +586,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         __builtin_amdgcn_sched_barrier(0);
         mfmas(1);
         __builtin_amdgcn_sched_barrier(0);
+        // The F0 reads above have had a whole MFMA group to land.  Waiting for them
+        // here, explicitly, keeps the compiler from putting a full LDS wait in front
+        // of the next MFMA group at the loop head (it cannot count reads across the
+        // back edge, and the 4-bit counter cannot express "all but the newest 16").
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0), vmcnt untouched
         if (FOLD && range_done) fold(cr);
         advance(cr, ck);
         buf = nbuf;
@@ -630,6 +636,7 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
             if (!fold) {
                 switch (wcfg) {
                     case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2>(p, batch, st);
+                    case 4: return launch_pipe_instance<256, 256, 2, 2, FMT, false, 2>(p, batch, st);
                     case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
                     case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
                     case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, false, 2>(p, batch, st);
