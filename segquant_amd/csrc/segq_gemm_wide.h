@@ -462,15 +462,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (int i = 0; i < B_IT; ++i) b_goff[i] = (uint32_t)min(n0 + s_row + i * RPI, p.N - 1) * (uint32_t)p.ldb + s_lc * 16;
     const int w_lds = wave * 8 * BK;
 
-    auto dma = [&](int r, int k, int buf) {
-        const uint8_t* ap = ((p.r[r].a_sel == 1) ? A2b : Ab) + k;
-        const uint8_t* bp = Bb + k;
-        uint8_t* as = As + buf * BM * BK + w_lds;
-        uint8_t* bs = Bs + buf * BN * BK + w_lds;
+    auto dma1 = [&](const uint8_t* ap, const uint8_t* bp, int buf, int i) {
+        if (i < A_IT) load16_to_lds(ap + a_goff[i], As + buf * BM * BK + w_lds + i * RPI * BK);
+        else load16_to_lds(bp + b_goff[i - A_IT], Bs + buf * BN * BK + w_lds + (i - A_IT) * RPI * BK);
+    };
+    auto dma = [&](const uint8_t* ap, const uint8_t* bp, int buf) {
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) load16_to_lds(ap + a_goff[i], as + i * RPI * BK);
-#pragma unroll
-        for (int i = 0; i < B_IT; ++i) load16_to_lds(bp + b_goff[i], bs + i * RPI * BK);
+        for (int i = 0; i < A_IT + B_IT; ++i) dma1(ap, bp, buf, i);
     };
 
     acc_t acc[TN][TM];
@@ -491,24 +489,17 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     const int b_frag = (wn * WN + lrow) * BK;
     frag_t fa[2][TM], fb[2][TN];
 
-    // K half h of the tile in buffer buf -> fragment slot h
-    auto frags = [&](int buf, int h) {
-        const uint8_t* as = As + buf * BM * BK + a_frag;
-        const uint8_t* bs = Bs + buf * BN * BK + b_frag;
+    // K half h of the tile in buffer buf -> fragment slot h, one 16-byte read at a
+    // time: reads 0 .. TM-1 are the activation fragments, TM .. TM+TN-1 the weights
+    auto frag1 = [&](int buf, int h, int i) {
         const int off = ((h * 4 + lgrp) ^ f_sw) << 4;
-#pragma unroll
-        for (int t = 0; t < TM; ++t) fa[h][t] = *reinterpret_cast<const v4i*>(as + t * 16 * BK + off);
-#pragma unroll
-        for (int t = 0; t < TN; ++t) fb[h][t] = *reinterpret_cast<const v4i*>(bs + t * 16 * BK + off);
+        if (i < TM) fa[h][i] = *reinterpret_cast<const v4i*>(As + buf * BM * BK + a_frag + i * 16 * BK + off);
+        else fb[h][i - TM] = *reinterpret_cast<const v4i*>(Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK + off);
     };
-    auto mfmas = [&](int h) {
+    auto frags = [&](int buf, int h) {
 #pragma unroll
-        for (int a = 0; a < TN; ++a)
-#pragma unroll
-            for (int b = 0; b < TM; ++b)
-                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[h][a], fa[h][b], acc[a][b], 0, 0, 0);
+        for (int i = 0; i < TM + TN; ++i) frag1(buf, h, i);
     };
-
     const int m_base = m0 + wm * WM + lrow;
     const int n_base = n0 + wn * WN + 4 * lgrp;
     auto fold = [&](int r) {
@@ -534,13 +525,20 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
     };
 
-    // (range, k) of the tile that is loaded two steps ahead of the one being multiplied
-    int lr = 0, lk = p.r[0].k0;
-    auto advance = [&](int& r, int& k) {
-        k += BK;
-        if (k >= p.r[r].k1) {
-            ++r;
-            k = (r < p.nr) ? p.r[r].k0 : 0;
+    // Two cursors walk the ranges: (lr, lk) is the tile loaded NS steps ahead,
+    // (cr, ck) the tile being multiplied.  The end of the current range and the
+    // source of its activations stay in registers, so the range table is read
+    // only when a cursor crosses into the next range.
+    int lr = 0, lk = p.r[0].k0, lk1 = p.r[0].k1;
+    const uint8_t* la = (p.r[0].a_sel == 1) ? A2b : Ab;
+    auto advance_load = [&]() {
+        lk += BK;
+        if (lk >= lk1) {
+            ++lr;
+            const int rr = min(lr, p.nr - 1);  // past the last range nothing more is loaded
+            lk = p.r[rr].k0;
+            lk1 = (lr < p.nr) ? p.r[rr].k1 : 0x7fffffff;
+            la = (p.r[rr].a_sel == 1) ? A2b : Ab;
         }
     };
     int steps = 0;
@@ -551,8 +549,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
 #pragma unroll
     for (int t = 0; t < NS; ++t) {
         if (t < steps) {
-            dma(lr, lk, t);
-            advance(lr, lk);
+            dma(la + lk, Bb + lk, t);
+            advance_load();
             ++issued;
         }
     }
@@ -562,39 +560,73 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     frags(0, 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop head must see F0 as landed on every path
 
-    int cr = 0, ck = p.r[0].k0;  // the tile being multiplied
-    int buf = 0;                  // its buffer, s % NS
-    for (int s = 0; s < steps; ++s) {
-        const bool last = s + 1 == steps;
-        const bool range_done = ck + BK >= p.r[cr].k1;
+    // One K step.  Fragment reads and DMA instructions are spread between the
+    // MFMAs: a wave issues in order, and an LDS or DMA instruction that has to
+    // queue holds up the MFMAs behind it, so a burst of them drains the matrix
+    // pipe of the whole SIMD (both its waves are in the same phase).  Issued one
+    // at a time they never queue.  DMA_ and MORE_ are compile-time so that the
+    // steady-state loop body has no branches.
+    int cr = 0, ck = p.r[0].k0, ck1 = p.r[0].k1;  // the tile being multiplied
+    int buf = 0;                                   // its buffer, s % NS
+    constexpr int NMF = TM * TN, NRD = TM + TN, NDM = A_IT + B_IT;
+    constexpr int RD_EVERY = (NMF >= 2 * NRD + 4) ? 2 : 1;
+    constexpr int DM_EVERY = (NMF / NDM > 1) ? NMF / NDM : 1;
+    static_assert(NRD * RD_EVERY <= NMF && NDM * DM_EVERY <= NMF, "more reads than MFMA slots");
+    auto step = [&](auto dma_c, auto more_c) {
+        constexpr bool DMA_ = decltype(dma_c)::value;
+        constexpr bool MORE_ = decltype(more_c)::value;
         const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
-        frags(buf, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(0);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int i = a * TM + b;
+                if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(buf, 1, i / RD_EVERY);
+                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
         // flight) and this wave's reads of tile s must be done, before anyone reads
         // tile s+1 or overwrites the buffer of tile s.
-        if (s + NS - 1 < steps) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * (A_IT + B_IT)));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(DMA_ ? (NS - 2) * NDM : 0));
         __syncthreads();
-        if (s + NS < steps) {  // tile s+NS goes where tile s was: both its halves are in registers
-            dma(lr, lk, buf);
-            advance(lr, lk);
-        }
-        if (!last) frags(nbuf, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(1);
-        __builtin_amdgcn_sched_barrier(0);
-        // The F0 reads above have had a whole MFMA group to land.  Waiting for them
-        // here, explicitly, keeps the compiler from putting a full LDS wait in front
-        // of the next MFMA group at the loop head (it cannot count reads across the
-        // back edge, and the 4-bit counter cannot express "all but the newest 16").
+        // tile s+NS goes where tile s was: both its halves are in registers
+        const uint8_t* const ap = la + lk;
+        const uint8_t* const bp = Bb + lk;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int i = a * TM + b;
+                if constexpr (DMA_) {
+                    if (i % DM_EVERY == DM_EVERY - 1 && i / DM_EVERY < NDM) dma1(ap, bp, buf, i / DM_EVERY);
+                }
+                if constexpr (MORE_) {
+                    if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(nbuf, 0, i / RD_EVERY);
+                }
+                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[1][a], fa[1][b], acc[a][b], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        // The reads of the next tile's first half have had most of an MFMA group to
+        // land.  Waiting for them here, explicitly, keeps the compiler from putting
+        // a full LDS wait in front of the first MFMA at the loop head (it cannot
+        // count reads across the back edge).
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0), vmcnt untouched
-        if (FOLD && range_done) fold(cr);
-        advance(cr, ck);
+        if constexpr (DMA_) advance_load();
+        ck += BK;
+        if (ck >= ck1) {  // the range is complete: fold it, move to the next one
+            if constexpr (FOLD) fold(cr);
+            ++cr;
+            const int rr = min(cr, p.nr - 1);
+            ck = p.r[rr].k0;
+            ck1 = p.r[rr].k1;
+        }
         buf = nbuf;
-    }
+    };
+    int s = 0;
+    for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
+    for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
+    if (s < steps) step(std::false_type{}, std::false_type{});
     wide_epilogue<BM, BN, WGM, WGN, FMT, false, FOLD>(p, acc, accf, smem, z, m0, n0, wave, lane);
 }
 
@@ -636,7 +668,6 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
             if (!fold) {
                 switch (wcfg) {
                     case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2>(p, batch, st);
-                    case 4: return launch_pipe_instance<256, 256, 2, 2, FMT, false, 2>(p, batch, st);
                     case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
                     case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
                     case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, false, 2>(p, batch, st);
