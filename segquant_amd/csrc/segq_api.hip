@@ -27,20 +27,34 @@ static bool is_float_dtype(int t) { return t == SEGQ_F32 || t == SEGQ_F16 || t =
 static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // Tile choice when the caller leaves it to the library.  The 8-wave kernels need
-// K in whole 128-byte steps and 32-bit row offsets.  Among their tiles the
-// 256 x 256 one moves the fewest operand bytes per MAC and wins as soon as it
-// occupies about two thirds of the CUs (measured on M = 4608: 216 tiles of
-// 256 x 256 beat 432 tiles of 256 x 128 by 30 %); below that, halve the tile.
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok) {
+// K in whole 128-byte steps and 32-bit row offsets.  A launch runs in rounds of
+// one tile per CU, so its time goes as rounds x tile area x a per-tile weight
+// (smaller tiles move more operand bytes per MAC: measured on M = 4608, 216
+// tiles of 256 x 256 beat 432 tiles of 256 x 128 by 30 %).  The 192 x 288 and
+// 288 x 192 tiles exist because 4608 rows of FLUX tokens make whole rounds with
+// them where 256 x 256 leaves the last round half empty.
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain_i8) {
     auto tiles = [&](int cfg) {
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
     };
-    if (wide_ok) {
-        const int first = FIRST_WIDE_CFG + (fold ? 1 : 0);  // no 256 x 256 with a second accumulator set
-        for (int cfg = first; cfg < FIRST_WIDE_CFG + 4; ++cfg)
-            if (tiles(cfg) >= 160) return cfg;
-        if (tiles(FIRST_WIDE_CFG + 3) >= 96) return FIRST_WIDE_CFG + 3;
+    if (wide_ok && tiles(FIRST_WIDE_CFG + 3) >= 96) {
+        static const double weight[6] = {1.0, 1.18, 1.18, 1.45, 1.04, 1.04};
+        const int64_t cus = 256;
+        int best = -1;
+        double best_cost = 0;
+        for (int i = 0; i < 6; ++i) {
+            if (i == 0 && fold) continue;                  // no 256 x 256 with a second accumulator set
+            if (i >= 4 && (fold || !plain_i8)) continue;  // plain int8 operands, one range only
+            const int cfg = FIRST_WIDE_CFG + i;
+            const int64_t rounds = (tiles(cfg) + cus - 1) / cus;
+            const double cost = (double)rounds * TILE_CFGS[cfg].bm * TILE_CFGS[cfg].bn * weight[i];
+            if (best < 0 || cost < best_cost) {
+                best = cfg;
+                best_cost = cost;
+            }
+        }
+        return best;
     }
     return tiles(2) >= 256 ? 2 : 3;
 }
@@ -111,7 +125,9 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     bool wide_ok = d->m * d->lda < (int64_t)1 << 32 && d->n * d->ldb < (int64_t)1 << 32;
     for (int i = 0; i < d->n_ranges; ++i) wide_ok = wide_ok && d->ranges[i].k_begin % 128 == 0 && d->ranges[i].k_len % 128 == 0;
     int cfg;
-    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok);
+    bool plain_i8 = i8;
+    for (int i = 0; i < d->n_ranges; ++i) plain_i8 = plain_i8 && d->ranges[i].a_sel < 2;
+    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok, plain_i8);
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
     if (cfg >= FIRST_WIDE_CFG) {

@@ -79,8 +79,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
         constexpr int RS = WN * 2 + 16;  // row stride in bytes; the 16 spreads rows over the banks
         __syncthreads();                 // the operand tiles are dead from here on
         uint8_t* patch = smem + wave * 16 * RS;
-        const int rd_row = lane / (WN / 8), rd_col = lane % (WN / 8);
-        constexpr int ROWS_PER_RD = 64 / (WN / 8);
+        constexpr int CH = WN / 8;  // 16-byte pieces per patch row
         float rwv[TN][4], bvv[TN][4];
 #pragma unroll
         for (int a = 0; a < TN; ++a) {
@@ -103,12 +102,14 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
             }
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for (int j = 0; j < 16 / ROWS_PER_RD; ++j) {
-                const int row = j * ROWS_PER_RD + rd_row;
-                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + rd_col * 16);
+            for (int j = 0; j < (16 * CH + 63) / 64; ++j) {
+                const int c = j * 64 + lane;
+                const int row = c / CH, col = c % CH;
+                if ((16 * CH) % 64 != 0 && c >= 16 * CH) continue;
+                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + col * 16);
                 const int m = m0 + wm * WM + b * 16 + row;
                 if (m < p.M)
-                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + rd_col * 8) = v;
+                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + col * 8) = v;
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -413,9 +414,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 16, TN = WN / 16;
-    constexpr int A_IT = BM * 8 / NT, B_IT = BN * 8 / NT;
-    constexpr int RPI = NT / 8;
-    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0 && RPI % 16 == 0, "tile does not divide over the threads");
+    constexpr int RPI = NT / 8;                                  // rows one pass of all threads covers
+    constexpr int A_IT = (BM + RPI - 1) / RPI, B_IT = (BN + RPI - 1) / RPI;
+    constexpr int A_TAIL = BM % RPI, B_TAIL = BN % RPI;          // rows of a last, partial pass (0: none)
+    static_assert(A_TAIL % 8 == 0 && B_TAIL % 8 == 0 && WM % 16 == 0 && WN % 16 == 0, "tile does not divide over the waves");
     typedef typename AccT<FMT>::type acc_t;
     static_assert(FMT == GEMM_I8, "two fragment sets per step: the 64-byte int8 MFMA");
     typedef v4i frag_t;
@@ -462,9 +464,30 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (int i = 0; i < B_IT; ++i) b_goff[i] = (uint32_t)min(n0 + s_row + i * RPI, p.N - 1) * (uint32_t)p.ldb + s_lc * 16;
     const int w_lds = wave * 8 * BK;
 
+    // a wave covers 8 rows of a pass, so whether it takes part in a partial last pass is wave-uniform
+    const bool a_skip = A_TAIL != 0 && wave * 8 >= A_TAIL;
+    const bool b_skip = B_TAIL != 0 && wave * 8 >= B_TAIL;
     auto dma1 = [&](const uint8_t* ap, const uint8_t* bp, int buf, int i) {
-        if (i < A_IT) load16_to_lds(ap + a_goff[i], As + buf * BM * BK + w_lds + i * RPI * BK);
-        else load16_to_lds(bp + b_goff[i - A_IT], Bs + buf * BN * BK + w_lds + (i - A_IT) * RPI * BK);
+        if (i < A_IT) {
+            if (i == A_IT - 1 && a_skip) return;
+            load16_to_lds(ap + a_goff[i], As + buf * BM * BK + w_lds + i * RPI * BK);
+        } else {
+            if (i == A_IT + B_IT - 1 && b_skip) return;
+            load16_to_lds(bp + b_goff[i - A_IT], Bs + buf * BN * BK + w_lds + (i - A_IT) * RPI * BK);
+        }
+    };
+    // "all but the newest nt tiles of this wave's DMA have landed, and all its LDS reads"
+    auto wait_dma = [&](auto nt_c) {
+        constexpr int nt = decltype(nt_c)::value;
+        constexpr int full = A_IT + B_IT;
+        if constexpr (nt == 0 || (A_TAIL == 0 && B_TAIL == 0)) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(nt * full));
+        } else {
+            const int miss = (a_skip ? 1 : 0) + (b_skip ? 1 : 0);
+            if (miss == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(nt * full));
+            else if (miss == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(nt * (full - 1)));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(nt * (full - 2)));
+        }
     };
     auto dma = [&](const uint8_t* ap, const uint8_t* bp, int buf) {
 #pragma unroll
@@ -554,8 +577,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             ++issued;
         }
     }
-    if (issued == NS) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * (A_IT + B_IT)));
-    else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+    if (issued == NS) wait_dma(std::integral_constant<int, NS - 1>{});
+    else wait_dma(std::integral_constant<int, 0>{});
     __syncthreads();
     frags(0, 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop head must see F0 as landed on every path
@@ -588,7 +611,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
         // flight) and this wave's reads of tile s must be done, before anyone reads
         // tile s+1 or overwrites the buffer of tile s.
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(DMA_ ? (NS - 2) * NDM : 0));
+        wait_dma(std::integral_constant<int, DMA_ ? NS - 2 : 0>{});
         __syncthreads();
         // tile s+NS goes where tile s was: both its halves are in registers
         const uint8_t* const ap = la + lk;
@@ -671,6 +694,8 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
                     case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
                     case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, false, 2>(p, batch, st);
+                    case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, false, 2>(p, batch, st);
+                    case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, false, 2>(p, batch, st);
                 }
             } else {
                 switch (wcfg) {
