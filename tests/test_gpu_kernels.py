@@ -221,6 +221,87 @@ def test_gemm_raw_accumulators(ops, tile, fa, fb, M, N, K):
         assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
 
 
+WIDE_TILES = [11, 12, 13, 14, 15, 16]   # the 8-wave kernels; 15 and 16 (192x288, 288x192) serve plain int8 only
+
+
+def _bf16_ulp(ref):
+    return np.abs(ref) * 2.0 ** -7 + 1e-30
+
+
+@pytest.mark.parametrize("tile", WIDE_TILES)
+@pytest.mark.parametrize("fa,fb", [(O.FMT_INT8, O.FMT_INT8), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_INT8, O.FMT_INT4)])
+@pytest.mark.parametrize("M,N,K", [(512, 576, 256), (300, 700, 384), (77, 130, 128)])
+def test_gemm_eight_wave_tiles(ops, tile, fa, fb, M, N, K):
+    """Raw accumulators (exact) and the fused bf16 epilogue (scales per row and per
+    column, bias; at most one bf16 unit from the oracle's single rounding) on
+    every 8-wave tile, on a shape of whole tiles and on ragged ones."""
+    a = _rand_codes((M, K), fa, 40)
+    b = _rand_codes((N, K), fb, 41)
+    ad, bd = _to_dev_codes(a, fa), _to_dev_codes(b, fb)
+    ldb = K // 2 if fb == O.FMT_INT4 else K
+    kw = dict(m=M, n=N, a_fmt=fa, b_fmt=fb, lda=K, ldb=ldb, tile=tile)
+    if tile >= 15 and fa != fb:
+        with pytest.raises(RuntimeError):
+            ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+        return
+    if tile >= 15 and fa != O.FMT_INT8:
+        with pytest.raises(RuntimeError):
+            ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+        return
+    ref = O.gemm_acc(a, b, fa, fb)
+    out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+    if fa == O.FMT_E4M3:
+        mag = np.abs(O.code_values(a, fa)) @ np.abs(O.code_values(b, fb)).T
+        assert (np.abs(out.cpu().numpy().astype(np.float64) - ref) <= FP8_ACC_TOL * mag + 1e-30).all()
+    else:
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
+    g = torch.Generator().manual_seed(42)
+    sx = torch.rand(M, generator=g) + 0.5
+    sw = torch.rand(N, generator=g) + 0.5
+    bias = torch.randn(N, generator=g)
+    y = ops.gemm(ad, bd, [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)], out_dtype=torch.bfloat16,
+                 bias=bias.to(DEV), **kw)
+    want = ref / (sx.numpy().astype(np.float64)[:, None] * sw.numpy().astype(np.float64)[None, :]) + bias.numpy()
+    got = y.float().cpu().numpy().astype(np.float64)
+    slack = FP8_ACC_TOL * mag / (sx.numpy()[:, None] * sw.numpy()[None, :]) if fa == O.FMT_E4M3 else 0.0
+    assert (np.abs(got - want) <= _bf16_ulp(want) + slack).all()
+
+
+@pytest.mark.parametrize("tile", [0, 11, 15, 16])
+def test_gemm_more_tiles_than_compute_units(ops, tile):
+    """4608 x 4608 outputs are 324 to 384 tiles, more than the 256 CUs hold at once."""
+    M, N, K = 4608, 4608, 256
+    a = _rand_codes((M, K), O.FMT_INT8, 43)
+    b = _rand_codes((N, K), O.FMT_INT8, 44)
+    ad, bd = _to_dev_codes(a, O.FMT_INT8), _to_dev_codes(b, O.FMT_INT8)
+    ref = O.gemm_acc(a, b, O.FMT_INT8, O.FMT_INT8)
+    kw = dict(m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT8, lda=K, ldb=K, tile=tile)
+    out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
+    g = torch.Generator().manual_seed(45)
+    sx = torch.rand(M, generator=g) + 0.5
+    sw = torch.rand(N, generator=g) + 0.5
+    bias = torch.randn(N, generator=g)
+    swn = sw.numpy().astype(np.float64)[None, :]
+    y = ops.gemm(ad, bd, [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)], out_dtype=torch.bfloat16,
+                 bias=bias.to(DEV), **kw)
+    want = ref / (sx.numpy().astype(np.float64)[:, None] * swn) + bias.numpy()
+    assert (np.abs(y.float().cpu().numpy().astype(np.float64) - want) <= _bf16_ulp(want)).all()
+    # two K segments with their own activation scales: the fp32 fold between ranges
+    sx2 = torch.rand(M, generator=g) + 0.5
+    rg = [ops.Range(0, 128, sx.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(128, 128, sx2.to(DEV), sw.to(DEV), 0, 1, 1)]
+    if tile >= 15:  # these tiles have no second accumulator set
+        with pytest.raises(RuntimeError):
+            ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **kw)
+        return
+    y = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **kw)
+    want = (O.gemm_acc(a[:, :128], b[:, :128], O.FMT_INT8, O.FMT_INT8) / (sx.numpy().astype(np.float64)[:, None] * swn)
+            + O.gemm_acc(a[:, 128:], b[:, 128:], O.FMT_INT8, O.FMT_INT8) / (sx2.numpy().astype(np.float64)[:, None] * swn)
+            + bias.numpy())
+    got = y.float().cpu().numpy().astype(np.float64)
+    assert (np.abs(got - want) <= _bf16_ulp(want) + 1e-5 * np.abs(want).max()).all()
+
+
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
 def test_gemm_sign_selected_halves_of_merged_codes(ops, fmt):
     M, N, K = 70, 90, 320
