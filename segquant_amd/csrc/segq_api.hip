@@ -154,6 +154,8 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
 
 using namespace segq;
 
+// only the C ABI leaves the library: everything else is built with hidden visibility
+#pragma GCC visibility push(default)
 extern "C" {
 
 int segq_version(void) { return 100; }
@@ -205,3 +207,4 @@ int segq_fake_e4m3(const void* x, void* out, int32_t dtype, int64_t numel, segq_
 }
 
 }  // extern "C"
+#pragma GCC visibility pop
