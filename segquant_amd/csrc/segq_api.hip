@@ -33,7 +33,7 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 // tiles of 256 x 256 beat 432 tiles of 256 x 128 by 30 %).  The 192 x 288 and
 // 288 x 192 tiles exist because 4608 rows of FLUX tokens make whole rounds with
 // them where 256 x 256 leaves the last round half empty.
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain_i8) {
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8) {
     auto tiles = [&](int cfg) {
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
@@ -45,7 +45,7 @@ static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide
         double best_cost = 0;
         for (int i = 0; i < 6; ++i) {
             if (i == 0 && fold) continue;                  // no 256 x 256 with a second accumulator set
-            if (i >= 4 && (fold || !plain_i8)) continue;  // plain int8 operands, one range only
+            if (i >= 4 && (fold || !plain8)) continue;  // plain int8 or e4m3 operands, one range only
             const int cfg = FIRST_WIDE_CFG + i;
             const int64_t rounds = (tiles(cfg) + cus - 1) / cus;
             const double cost = (double)rounds * TILE_CFGS[cfg].bm * TILE_CFGS[cfg].bn * weight[i];
@@ -125,9 +125,9 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     bool wide_ok = d->m * d->lda < (int64_t)1 << 32 && d->n * d->ldb < (int64_t)1 << 32;
     for (int i = 0; i < d->n_ranges; ++i) wide_ok = wide_ok && d->ranges[i].k_begin % 128 == 0 && d->ranges[i].k_len % 128 == 0;
     int cfg;
-    bool plain_i8 = i8;
-    for (int i = 0; i < d->n_ranges; ++i) plain_i8 = plain_i8 && d->ranges[i].a_sel < 2;
-    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok, plain_i8);
+    bool plain8 = i8 || f8;  // both operands straight to LDS: no sign selection, no int4 unpacking
+    for (int i = 0; i < d->n_ranges; ++i) plain8 = plain8 && d->ranges[i].a_sel < 2;
+    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok, plain8);
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
     if (cfg >= FIRST_WIDE_CFG) {

@@ -419,11 +419,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     constexpr int A_TAIL = BM % RPI, B_TAIL = BN % RPI;          // rows of a last, partial pass (0: none)
     static_assert(A_TAIL % 8 == 0 && B_TAIL % 8 == 0 && WM % 16 == 0 && WN % 16 == 0, "tile does not divide over the waves");
     typedef typename AccT<FMT>::type acc_t;
-    static_assert(FMT == GEMM_I8, "two fragment sets per step: the 64-byte int8 MFMA");
-    typedef v4i frag_t;
+    constexpr bool F8 = FMT == GEMM_F8;
     const acc_t acc_zero = {0, 0, 0, 0};
 
     static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
+    static_assert(!F8 || (NS == 2 && TN >= 3), "the e4m3 schedule reads two weight fragments ahead in a two-stage ring");
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t* const As = smem;                  // [NS][BM][128]
     uint8_t* const Bs = smem + NS * BM * BK;   // [NS][BN][128]
@@ -510,14 +510,32 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     const int f_sw = swz(lrow);
     const int a_frag = (wm * WM + lrow) * BK;
     const int b_frag = (wn * WN + lrow) * BK;
-    frag_t fa[2][TM], fb[2][TN];
+    // int8: two fragment sets, one per 64-byte K half of a step.  e4m3: one set of
+    // 32-byte fragments (the 16 x 16 x 128 MFMA eats a whole step), whose registers
+    // are refilled for the next step as the current one lets go of them.
+    v4i fa[F8 ? 1 : 2][F8 ? 1 : TM], fb[F8 ? 1 : 2][F8 ? 1 : TN];
+    v8i fa8[F8 ? TM : 1], fb8[F8 ? TN : 1];
+    auto frag8 = [&](int buf, int i) {  // fragment i of the step in buffer buf: 0 .. TM-1 activations, then weights
+      if constexpr (F8) {
+        const int off0 = ((2 * lgrp) ^ f_sw) << 4;
+        const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
+        const uint8_t* src = (i < TM) ? As + buf * BM * BK + a_frag + i * 16 * BK : Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK;
+        const v4i lo = *reinterpret_cast<const v4i*>(src + off0);
+        const v4i hi = *reinterpret_cast<const v4i*>(src + off1);
+        const v8i f = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if (i < TM) fa8[i] = f;
+        else fb8[i - TM] = f;
+      }
+    };
 
     // K half h of the tile in buffer buf -> fragment slot h, one 16-byte read at a
     // time: reads 0 .. TM-1 are the activation fragments, TM .. TM+TN-1 the weights
     auto frag1 = [&](int buf, int h, int i) {
-        const int off = ((h * 4 + lgrp) ^ f_sw) << 4;
-        if (i < TM) fa[h][i] = *reinterpret_cast<const v4i*>(As + buf * BM * BK + a_frag + i * 16 * BK + off);
-        else fb[h][i - TM] = *reinterpret_cast<const v4i*>(Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK + off);
+        if constexpr (!F8) {
+            const int off = ((h * 4 + lgrp) ^ f_sw) << 4;
+            if (i < TM) fa[h][i] = *reinterpret_cast<const v4i*>(As + buf * BM * BK + a_frag + i * 16 * BK + off);
+            else fb[h][i - TM] = *reinterpret_cast<const v4i*>(Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK + off);
+        }
     };
     auto frags = [&](int buf, int h) {
 #pragma unroll
@@ -580,8 +598,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     if (issued == NS) wait_dma(std::integral_constant<int, NS - 1>{});
     else wait_dma(std::integral_constant<int, 0>{});
     __syncthreads();
-    frags(0, 0);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop head must see F0 as landed on every path
+    if constexpr (F8) {
+#pragma unroll
+        for (int i = 0; i <= TM; ++i) frag8(0, i);  // activations and the first weight fragment
+    } else {
+        frags(0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop head must see them as landed on every path
 
     // One K step.  Fragment reads and DMA instructions are spread between the
     // MFMAs: a wave issues in order, and an LDS or DMA instruction that has to
@@ -595,7 +618,66 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     constexpr int RD_EVERY = (NMF >= 2 * NRD + 4) ? 2 : 1;
     constexpr int DM_EVERY = (NMF / NDM > 1) ? NMF / NDM : 1;
     static_assert(NRD * RD_EVERY <= NMF && NDM * DM_EVERY <= NMF, "more reads than MFMA slots");
-    auto step = [&](auto dma_c, auto more_c) {
+    // e4m3 schedule of one step.  On entry the activation fragments and weight
+    // fragment 0 are in registers.  Column block a reads weight fragment a + 2
+    // (block 0 also fragment 1), so after block TN - 3 every read of this step is
+    // issued; there the step has its barrier.  The last two blocks refill the
+    // registers this step is done with: next weight fragment 0, then each
+    // activation fragment right behind the last MFMA that reads it, with the DMA
+    // of step s + 2 spread over the same MFMAs.
+    auto step8 = [&](auto dma_c, auto more_c) {
+        constexpr bool DMA_ = decltype(dma_c)::value;
+        constexpr bool MORE_ = decltype(more_c)::value;
+        constexpr int NDM8 = A_IT + B_IT, TAIL = 2 * TM;  // DMA instructions over the tail's MFMAs
+        const int nbuf = buf ^ 1;
+#pragma unroll
+        for (int a = 0; a < TN - 2; ++a) {
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                if (b == 0 && a == 0) frag8(buf, TM + 1);
+                if (b == (TM > 1 ? 1 : 0)) frag8(buf, TM + a + 2);
+                acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        wait_dma(std::integral_constant<int, 0>{});
+        __syncthreads();
+        const uint8_t* const ap = la + lk;
+        const uint8_t* const bp = Bb + lk;
+#pragma unroll
+        for (int a = TN - 2; a < TN; ++a) {
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+                const int j = (a - (TN - 2)) * TM + b;
+                if constexpr (DMA_) {
+#pragma unroll
+                    for (int i = j * NDM8 / TAIL; i < (j + 1) * NDM8 / TAIL; ++i) dma1(ap, bp, buf, i);
+                }
+                if constexpr (MORE_) {
+                    if (a == TN - 2 && b == 0) frag8(nbuf, TM);  // next weight fragment 0: its registers were free since block 0
+                    if (a == TN - 1) frag8(nbuf, b);              // next activation fragment b: this was its last reader
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // A full LDS wait: the last activation fragments were read a few MFMAs ago
+        // and this exposes part of their latency, but with reads still in flight
+        // over the loop's back edge the compiler puts the same wait in front of the
+        // next step's second MFMA, behind that step's first reads.
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        if constexpr (DMA_) advance_load();
+        ck += BK;
+        if (ck >= ck1) {
+            if constexpr (FOLD) fold(cr);
+            ++cr;
+            const int rr = min(cr, p.nr - 1);
+            ck = p.r[rr].k0;
+            ck1 = p.r[rr].k1;
+        }
+        buf = nbuf;
+    };
+    auto step_i8 = [&](auto dma_c, auto more_c) {
         constexpr bool DMA_ = decltype(dma_c)::value;
         constexpr bool MORE_ = decltype(more_c)::value;
         const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
@@ -646,6 +728,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
         buf = nbuf;
     };
+    auto step = [&](auto dma_c, auto more_c) {
+        if constexpr (F8) step8(dma_c, more_c);
+        else step_i8(dma_c, more_c);
+    };
     int s = 0;
     for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
     for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
@@ -686,14 +772,15 @@ int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 
 template <int FMT, bool B4>
 int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st) {
-    if constexpr (FMT == GEMM_I8 && !B4) {
-        if (!asel) {  // plain int8 operands: the software-pipelined kernel
+    if constexpr (!B4) {
+        constexpr bool F8W = FMT == GEMM_F8;  // the e4m3 schedule wants three or more column blocks per wave
+        if (!asel) {  // plain 8-bit operands, both straight to LDS: the software-pipelined kernel
             if (!fold) {
                 switch (wcfg) {
                     case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2>(p, batch, st);
                     case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
                     case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
-                    case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, false, 2>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, F8W ? 4 : 2, F8W ? 2 : 4, FMT, false, 2>(p, batch, st);
                     case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, false, 2>(p, batch, st);
                     case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, false, 2>(p, batch, st);
                 }
@@ -701,7 +788,7 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                 switch (wcfg) {
                     case 0: case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2>(p, batch, st);
                     case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2>(p, batch, st);
-                    case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, true, 2>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, F8W ? 4 : 2, F8W ? 2 : 4, FMT, true, 2>(p, batch, st);
                 }
             }
         }
