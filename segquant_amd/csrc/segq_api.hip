@@ -33,7 +33,7 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 // tiles of 256 x 256 beat 432 tiles of 256 x 128 by 30 %).  The 192 x 288 and
 // 288 x 192 tiles exist because 4608 rows of FLUX tokens make whole rounds with
 // them where 256 x 256 leaves the last round half empty.
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8) {
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8) {  // fold: needs a second accumulator set
     auto tiles = [&](int cfg) {
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
@@ -127,12 +127,15 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     int cfg;
     bool plain8 = i8 || f8;  // both operands straight to LDS: no sign selection, no int4 unpacking
     for (int i = 0; i < d->n_ranges; ++i) plain8 = plain8 && d->ranges[i].a_sel < 2;
-    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold, wide_ok, plain8);
+    // several ranges cost a second (fp32) accumulator set, and with it the biggest tiles,
+    // unless the accumulators are fp32 already (plain e4m3: rescaled in place)
+    const bool fold2 = fold && !(f8 && plain8);
+    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
     if (cfg >= FIRST_WIDE_CFG) {
         if (!wide_ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs K ranges in multiples of 128", cfg + 1);
-        if (fold && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
+        if (fold2 && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
     } else if (cfg >= FIRST_BIG_CFG) {
         if (!wide_ok || w4 || fold)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs one range, 8-bit weights and K in multiples of 128", cfg + 1);

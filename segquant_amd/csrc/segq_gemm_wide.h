@@ -26,7 +26,7 @@ namespace segq {
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
 __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT<FMT>::type (&acc)[BN / WGN / 16][BM / WGM / 16],
                                               v4f (&accf)[FOLD ? BN / WGN / 16 : 1][FOLD ? BM / WGM / 16 : 1],
-                                              uint8_t* smem, int64_t z, int m0, int n0, int wave, int lane) {
+                                              uint8_t* smem, int64_t z, int m0, int n0, int wave, int lane, int r_epi = 0) {
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 16, TN = WN / 16;
     typedef typename AccT<FMT>::type acc_t;
@@ -71,7 +71,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
     }
 
     float rx[TM];
-    if constexpr (!FOLD) range_rx(0, rx);
+    if constexpr (!FOLD) range_rx(r_epi, rx);  // the range whose scales the accumulators are in units of
     const bool is16 = p.out_dtype != SEGQ_F32;
     const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
     if (via_lds) {
@@ -83,7 +83,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
         float rwv[TN][4], bvv[TN][4];
 #pragma unroll
         for (int a = 0; a < TN; ++a) {
-            if constexpr (!FOLD) range_rw(0, a, rwv[a]);
+            if constexpr (!FOLD) range_rw(r_epi, a, rwv[a]);
 #pragma unroll
             for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
         }
@@ -118,7 +118,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
 #pragma unroll
     for (int a = 0; a < TN; ++a) {
         float rw[4];
-        if constexpr (!FOLD) range_rw(0, a, rw);
+        if constexpr (!FOLD) range_rw(r_epi, a, rw);
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (p.bias) {
 #pragma unroll
@@ -420,6 +420,12 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     static_assert(A_TAIL % 8 == 0 && B_TAIL % 8 == 0 && WM % 16 == 0 && WN % 16 == 0, "tile does not divide over the waves");
     typedef typename AccT<FMT>::type acc_t;
     constexpr bool F8 = FMT == GEMM_F8;
+    // Several ranges: int32 accumulators are folded into a second, fp32 set at the
+    // end of each range.  fp32 accumulators (e4m3) need no second set: at a range
+    // boundary they are rescaled from the finished range's scales to the next
+    // one's (acc *= sx' sw' / (sx sw), one fp32 rounding), so the sum stays in
+    // units of the current range and the epilogue divides by the last range's.
+    constexpr bool ACCF = FOLD && !F8;
     const acc_t acc_zero = {0, 0, 0, 0};
 
     static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
@@ -495,12 +501,12 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     };
 
     acc_t acc[TN][TM];
-    v4f accf[FOLD ? TN : 1][FOLD ? TM : 1];
+    v4f accf[ACCF ? TN : 1][ACCF ? TM : 1];
 #pragma unroll
     for (int a = 0; a < TN; ++a)
 #pragma unroll
         for (int b = 0; b < TM; ++b) acc[a][b] = acc_zero;
-    if constexpr (FOLD) {
+    if constexpr (ACCF) {
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
@@ -544,7 +550,33 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     const int m_base = m0 + wm * WM + lrow;
     const int n_base = n0 + wn * WN + 4 * lgrp;
     auto fold = [&](int r) {
-        if constexpr (FOLD) {
+        if constexpr (FOLD && F8) {
+            if (r + 1 < p.nr) {  // rescale to the next range's units
+                const float* sx = p.r[r].sx + z * p.bsSx;
+                const float* sw = p.r[r].sw + z * p.bsSw;
+                const float* sx2 = p.r[r + 1].sx + z * p.bsSx;
+                const float* sw2 = p.r[r + 1].sw + z * p.bsSw;
+                const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs, rs2 = p.r[r + 1].sx_rs, cs2 = p.r[r + 1].sw_cs;
+                float fx[TM];
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    const int64_t m = min(m_base + b * 16, p.M - 1);
+                    fx[b] = sx2[m * rs2] * __builtin_amdgcn_rcpf(sx[m * rs]);
+                }
+#pragma unroll
+                for (int a = 0; a < TN; ++a) {
+                    v4f fw;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int64_t n = min(n_base + a * 16 + v, p.N - 1);
+                        fw[v] = sw2[n * cs2] * __builtin_amdgcn_rcpf(sw[n * cs]);
+                    }
+#pragma unroll
+                    for (int b = 0; b < TM; ++b) acc[a][b] = acc[a][b] * (fw * fx[b]);
+                }
+            }
+        }
+        if constexpr (ACCF) {
             const float* sx = p.r[r].sx + z * p.bsSx;
             const float* sw = p.r[r].sw + z * p.bsSw;
             const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs;
@@ -736,7 +768,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
     for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
     if (s < steps) step(std::false_type{}, std::false_type{});
-    wide_epilogue<BM, BN, WGM, WGN, FMT, false, FOLD>(p, acc, accf, smem, z, m0, n0, wave, lane);
+    wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, ACCF ? 0 : p.nr - 1);
 }
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
@@ -783,6 +815,15 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 3: return launch_pipe_instance<128, 128, F8W ? 4 : 2, F8W ? 2 : 4, FMT, false, 2>(p, batch, st);
                     case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, false, 2>(p, batch, st);
                     case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, false, 2>(p, batch, st);
+                }
+            } else if constexpr (F8W) {  // fp32 accumulators are rescaled in place: every tile serves several ranges
+                switch (wcfg) {
+                    case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, true, 2>(p, batch, st);
+                    case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2>(p, batch, st);
+                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, 4, 2, FMT, true, 2>(p, batch, st);
+                    case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, true, 2>(p, batch, st);
+                    case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, true, 2>(p, batch, st);
                 }
             } else {
                 switch (wcfg) {
