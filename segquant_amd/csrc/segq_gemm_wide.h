@@ -26,7 +26,8 @@ namespace segq {
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
 __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT<FMT>::type (&acc)[BN / WGN / 16][BM / WGM / 16],
                                               v4f (&accf)[FOLD ? BN / WGN / 16 : 1][FOLD ? BM / WGM / 16 : 1],
-                                              uint8_t* smem, int64_t z, int m0, int n0, int wave, int lane, int r_epi = 0) {
+                                              uint8_t* smem, int64_t z, int m0, int n0, int wave, int lane, int r_epi = 0,
+                                              const float* epi = nullptr) {
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 16, TN = WN / 16;
     typedef typename AccT<FMT>::type acc_t;
@@ -70,10 +71,18 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
         return;
     }
 
-    float rx[TM];
-    if constexpr (!FOLD) range_rx(r_epi, rx);  // the range whose scales the accumulators are in units of
     const bool is16 = p.out_dtype != SEGQ_F32;
     const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
+    float rx[TM];
+    // epi: the tile's vectors parked in LDS by the caller, [1/sx BM | 1/sw BN | bias BN]
+    if constexpr (!FOLD) {
+        if (via_lds && epi) {
+#pragma unroll
+            for (int b = 0; b < TM; ++b) rx[b] = epi[wm * WM + b * 16 + lrow];
+        } else {
+            range_rx(r_epi, rx);  // the range whose scales the accumulators are in units of
+        }
+    }
     if (via_lds) {
         // every wave transposes 16 rows at a time through its own patch of LDS
         constexpr int RS = WN * 2 + 16;  // row stride in bytes; the 16 spreads rows over the banks
@@ -81,11 +90,24 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
         uint8_t* patch = smem + wave * 16 * RS;
         constexpr int CH = WN / 8;  // 16-byte pieces per patch row
         float rwv[TN][4], bvv[TN][4];
+        if (epi) {
 #pragma unroll
-        for (int a = 0; a < TN; ++a) {
-            if constexpr (!FOLD) range_rw(r_epi, a, rwv[a]);
+            for (int a = 0; a < TN; ++a) {
+                const v4f w = *reinterpret_cast<const v4f*>(epi + BM + wn * WN + a * 16 + 4 * lgrp);
+                const v4f bb = *reinterpret_cast<const v4f*>(epi + BM + BN + wn * WN + a * 16 + 4 * lgrp);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
+                for (int v = 0; v < 4; ++v) {
+                    rwv[a][v] = w[v];
+                    bvv[a][v] = bb[v];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                if constexpr (!FOLD) range_rw(r_epi, a, rwv[a]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
+            }
         }
 #pragma unroll
         for (int b = 0; b < TM; ++b) {
@@ -617,6 +639,30 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     int steps = 0;
     for (int i = 0; i < p.nr; ++i) steps += (p.r[i].k1 - p.r[i].k0) / BK;
 
+    // The epilogue's vectors (1/sx per row, 1/sw and bias per column of this tile)
+    // are fetched first of all, so that the wait for the first DMA covers them, and
+    // parked in LDS behind the stages: the epilogue then starts without a round
+    // trip to memory, and without the ~70 small loads per wave it would take there.
+    constexpr int EPI_FLOATS = BM + 2 * BN, EPI_IT = (EPI_FLOATS + NT - 1) / NT;
+    float* const epi = reinterpret_cast<float*>(smem + NS * (BM + BN) * BK);
+    const int r_epi = ACCF ? 0 : p.nr - 1;  // the range whose units the accumulators end up in
+    float epi_val[EPI_IT];
+    const bool want_epi = p.out_dtype != SEGQ_ACC;  // raw accumulators come with no scales at all (null pointers)
+#pragma unroll
+    for (int i = 0; i < EPI_IT; ++i) {
+        const int e = i * NT + tid;
+        float v = 0.0f;
+        if (!want_epi) {
+        } else if (e < BM) {
+            if constexpr (!ACCF) v = (p.r[r_epi].sx + z * p.bsSx)[(int64_t)min(m0 + e, p.M - 1) * p.r[r_epi].sx_rs];
+        } else if (e < BM + BN) {
+            if constexpr (!ACCF) v = (p.r[r_epi].sw + z * p.bsSw)[(int64_t)min(n0 + e - BM, p.N - 1) * p.r[r_epi].sw_cs];
+        } else if (e < EPI_FLOATS) {
+            if (p.bias) v = load_bias(p.bias, p.bias_dtype, min(n0 + e - BM - BN, p.N - 1));
+        }
+        epi_val[i] = v;
+    }
+
     // prologue: tiles 0 .. NS-1 on their way into buffers 0 .. NS-1; wait for tile 0
     int issued = 0;
 #pragma unroll
@@ -629,6 +675,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     }
     if (issued == NS) wait_dma(std::integral_constant<int, NS - 1>{});
     else wait_dma(std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int i = 0; i < EPI_IT; ++i) {
+        const int e = i * NT + tid;
+        if (e < EPI_FLOATS) epi[e] = (e < BM + BN && !ACCF) ? __builtin_amdgcn_rcpf(epi_val[i]) : epi_val[i];
+    }
     __syncthreads();
     if constexpr (F8) {
 #pragma unroll
@@ -768,7 +819,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
     for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
     if (s < steps) step(std::false_type{}, std::false_type{});
-    wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, ACCF ? 0 : p.nr - 1);
+    wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, r_epi, epi);
 }
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
@@ -790,7 +841,7 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS>
 int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS>;
-    constexpr int lds = NS * (BM + BN) * BK;
+    constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4;  // the stages and the epilogue's vectors
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
