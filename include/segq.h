@@ -181,6 +181,14 @@ typedef struct segq_gemm_desc {
     int64_t batch_stride_sw;  /* floats, applied to every range's sw */
     int32_t n_ranges;   /* 1 .. SEGQ_MAX_RANGES */
     int32_t tile;       /* 0 = choose; otherwise a tile configuration id, see segq_gemm_tile_count */
+    void* workspace;    /* device or NULL.  With int4 weights and at least batch * n * Kp bytes here (Kp = the
+                         * largest range end rounded up to 16), b is first expanded to int8 in the workspace by
+                         * a small kernel and the int8 GEMM kernels run on that (same accumulators, bit for bit;
+                         * worth it when m is large and the GEMM is bound by the matrix cores, not by reading b).
+                         * NULL or too small: int4 weights are unpacked on their way into LDS inside the GEMM.
+                         * Contents are undefined afterwards.  Replaces nothing in the reference, whose CUTLASS
+                         * kernel converts int4 in registers (segquant/src/real_quant/real_gemm.cu:208-305). */
+    int64_t workspace_bytes;
     segq_krange ranges[SEGQ_MAX_RANGES];
 } segq_gemm_desc;
 

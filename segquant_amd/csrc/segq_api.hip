@@ -59,6 +59,30 @@ static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide
     return tiles(2) >= 256 ? 2 : 3;
 }
 
+// int4 weight rows (two values per byte, even k in the low nibble) -> int8 rows.
+// One thread expands 16 packed bytes to 32 values.
+__global__ void __launch_bounds__(256) expand_i4_kernel(const uint8_t* src, int64_t ld_src, uint8_t* dst, int64_t ld_dst,
+                                                        int64_t rows, int64_t chunks_per_row) {
+    const int64_t total = rows * chunks_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / chunks_per_row, c = i - row * chunks_per_row;
+        const uint4 v = *reinterpret_cast<const uint4*>(src + row * ld_src + c * 16);
+        const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+        uint32_t out[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t e = in[j] & 0x0F0F0F0Fu, o = (in[j] >> 4) & 0x0F0F0F0Fu;
+            e |= (e & 0x08080808u) * 0x1Eu;  // sign-extend each nibble into its byte
+            o |= (o & 0x08080808u) * 0x1Eu;
+            out[2 * j] = __builtin_amdgcn_perm(o, e, 0x05010400u);      // k0 k1 k2 k3
+            out[2 * j + 1] = __builtin_amdgcn_perm(o, e, 0x07030602u);  // k4 k5 k6 k7
+        }
+        uint4* q = reinterpret_cast<uint4*>(dst + row * ld_dst + c * 32);
+        q[0] = make_uint4(out[0], out[1], out[2], out[3]);
+        q[1] = make_uint4(out[4], out[5], out[6], out[7]);
+    }
+}
+
 static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     if (!d) return fail(SEGQ_ERR_ARG, "segq_gemm: null descriptor");
     if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
@@ -108,6 +132,31 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     // int4 weights are staged as value*16: keep |acc| below 2^31
     if (w4 && ktotal > 131071) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: K too large for int4 weights");
     if (kmax > 0x7fffff00) return fail(SEGQ_ERR_ARG, "segq_gemm: K too large");
+
+    if (w4 && d->workspace) {
+        // expand b to int8 in the caller's workspace and run the int8 kernels on it
+        const int64_t kp = (kmax + 31) & ~(int64_t)31;  // whole 16-byte packed chunks
+        if (al(d->workspace, 16) && d->workspace_bytes >= d->batch * d->n * kp && kp / 2 <= d->ldb) {
+            const int64_t chunks = kp / 32;
+            for (int64_t zb = 0; zb < d->batch; ++zb) {
+                const int64_t total = d->n * chunks;
+                const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+                hipLaunchKernelGGL(expand_i4_kernel, dim3(blocks), dim3(256), 0, st,
+                                   static_cast<const uint8_t*>(d->b) + zb * d->batch_stride_b, d->ldb,
+                                   static_cast<uint8_t*>(d->workspace) + zb * d->n * kp, kp, d->n, chunks);
+            }
+            const int rc = check_launch("segq_gemm (int4 expansion)");
+            if (rc != SEGQ_OK) return rc;
+            segq_gemm_desc d8 = *d;
+            d8.b_fmt = SEGQ_CODE_I8;
+            d8.b = d->workspace;
+            d8.ldb = kp;
+            d8.batch_stride_b = d->n * kp;
+            d8.workspace = nullptr;
+            d8.workspace_bytes = 0;
+            return gemm_impl(&d8, st);
+        }
+    }
 
     p.A = static_cast<const uint8_t*>(d->a);
     p.A2 = static_cast<const uint8_t*>(d->a_neg);

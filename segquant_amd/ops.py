@@ -156,15 +156,31 @@ class Range:
     sw_col_stride: int = 0
 
 
+_int4_ws = {}
+
+
+def int4_workspace(device, nbytes: int) -> torch.Tensor:
+    """A per-device scratch tensor of at least ``nbytes`` for expanded int4 weights,
+    grown on demand and shared by every layer (launches on one stream run in order,
+    and its contents only live for the duration of one GEMM launch)."""
+    key = torch.device(device)
+    ws = _int4_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=key)
+        _int4_ws[key] = ws
+    return ws
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
          out_dtype, lda: int, ldb: int, a_neg: Optional[torch.Tensor] = None,
          bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
-         tile: int = 0) -> torch.Tensor:
+         tile: int = 0, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
-    accumulators (int32 for integer codes, float32 for e4m3).
+    accumulators (int32 for integer codes, float32 for e4m3).  ``workspace``: a
+    byte tensor the library may expand int4 weights into (see ``int4_workspace``).
     """
     _need_cuda(a, b, a_neg, bias)
     raw = out_dtype == "acc"
@@ -190,6 +206,9 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
     if not 1 <= len(ranges) <= L.SEGQ_MAX_RANGES:
         raise RuntimeError(f"1..{L.SEGQ_MAX_RANGES} ranges")
     d.n_ranges = len(ranges); d.tile = tile
+    if workspace is not None:
+        _need_cuda(workspace)
+        d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()
     for i, r in enumerate(ranges):
         kr = d.ranges[i]
         kr.k_begin = r.k_begin; kr.k_len = r.k_len; kr.a_sel = r.a_sel

@@ -55,13 +55,16 @@ def _dev(c, fmt):
 
 
 @pytest.mark.parametrize("name,M,K,N", SHAPES)
-@pytest.mark.parametrize("fb", [O.FMT_INT8, O.FMT_INT4])
-def test_full_size_integer_accumulators_product_check(ops, name, M, K, N, fb):
+@pytest.mark.parametrize("fb,lend", [(O.FMT_INT8, False), (O.FMT_INT4, False), (O.FMT_INT4, True)])
+def test_full_size_integer_accumulators_product_check(ops, name, M, K, N, fb, lend):
+    """lend: int4 weights expanded into a workspace the caller lends (the int8 kernels
+    run); otherwise unpacked inside the GEMM."""
     a = _codes((M, K), O.FMT_INT8, 100)
     b = _codes((N, K), fb, 101)
     ldb = K // 2 if fb == O.FMT_INT4 else K
+    ws = ops.int4_workspace(DEV, N * K) if lend else None
     out = ops.gemm(_dev(a, O.FMT_INT8), _dev(b, fb), [ops.Range(0, K, None, None)], m=M, n=N, a_fmt=O.FMT_INT8,
-                   b_fmt=fb, out_dtype="acc", lda=K, ldb=ldb)
+                   b_fmt=fb, out_dtype="acc", lda=K, ldb=ldb, workspace=ws)
     c = out.cpu().numpy().astype(np.int64)
     g = np.random.default_rng(102)
     a64, b64 = a.astype(np.int64), b.astype(np.int64)

@@ -298,6 +298,34 @@ def test_gemm_more_tiles_than_compute_units(ops, tile):
     assert (np.abs(got - want) <= _bf16_ulp(want) + 1e-5 * np.abs(want).max()).all()
 
 
+def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
+    """With a workspace the int4 weights are expanded to int8 first: same accumulators
+    bit for bit as unpacking inside the GEMM, ragged shapes, a batch, K segments with
+    a sign-selected DualScale range, and a workspace that is too small (ignored)."""
+    M, N, K, Z = 200, 300, 416, 2
+    a = np.stack([_rand_codes((M, K), O.FMT_INT8, 70 + z) for z in range(Z)])
+    b = np.stack([_rand_codes((N, K), O.FMT_INT4, 80 + z) for z in range(Z)])
+    ad = torch.stack([_to_dev_codes(a[z], O.FMT_INT8) for z in range(Z)])
+    bd = torch.stack([_to_dev_codes(b[z], O.FMT_INT4) for z in range(Z)])
+    kw = dict(m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT4, lda=K, ldb=K // 2, batch=Z, batch_stride_a=M * K,
+              batch_stride_b=N * K // 2)
+    ws = torch.empty(Z * N * K, dtype=torch.uint8, device=DEV)
+    fused = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+    lent = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", workspace=ws, **kw)
+    small = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", workspace=ws[:100], **kw)
+    assert torch.equal(fused, lent) and torch.equal(fused, small)
+    for z in range(Z):
+        assert np.array_equal(lent[z].cpu().numpy().astype(np.int64), O.gemm_acc(a[z], b[z], O.FMT_INT8, O.FMT_INT4).astype(np.int64))
+    g = torch.Generator().manual_seed(90)
+    sx, sx2, sw, bias = (torch.rand(M, generator=g) + 0.5).to(DEV), (torch.rand(M, generator=g) + 0.5).to(DEV), \
+        (torch.rand(N, generator=g) + 0.5).to(DEV), torch.randn(N, generator=g).to(DEV)
+    rg = [ops.Range(0, 128, sx, sw, 0, 1, 1), ops.Range(128, K - 128, sx2, sw, 2, 1, 1), ops.Range(128, K - 128, sx, sw, 3, 1, 1)]
+    kw1 = dict(kw, batch=1, batch_stride_a=0, batch_stride_b=0)
+    y0 = ops.gemm(ad[0], bd[0], rg, out_dtype=torch.float32, bias=bias, **kw1)
+    y1 = ops.gemm(ad[0], bd[0], rg, out_dtype=torch.float32, bias=bias, workspace=ws, **kw1)
+    assert (y0 - y1).abs().max().item() <= 2e-6 * y0.abs().max().item()
+
+
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
 def test_gemm_sign_selected_halves_of_merged_codes(ops, fmt):
     M, N, K = 70, 90, 320
