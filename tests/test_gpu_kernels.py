@@ -261,6 +261,32 @@ def test_gemm_eight_wave_tiles(ops, tile, fa, fb, M, N, K):
     got = y.float().cpu().numpy().astype(np.float64)
     slack = FP8_ACC_TOL * mag / (sx.numpy()[:, None] * sw.numpy()[None, :]) if fa == O.FMT_E4M3 else 0.0
     assert (np.abs(got - want) <= _bf16_ulp(want) + slack).all()
+    # two K ranges with their own activation and weight scales: int32 accumulators are
+    # folded into fp32 ones (not on the 192x288 / 288x192 tiles), fp32 accumulators
+    # are rescaled in place at the boundary (every tile)
+    K0 = 128
+    if K <= K0:
+        return
+    sx2 = torch.rand(M, generator=g) + 0.5
+    sw2 = torch.rand(N, generator=g) + 0.5
+    rg = [ops.Range(0, K0, sx.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(K0, K - K0, sx2.to(DEV), sw2.to(DEV), 0, 1, 1)]
+    if tile >= 15 and fa == O.FMT_INT8:
+        with pytest.raises(RuntimeError):
+            ops.gemm(ad, bd, rg, out_dtype=torch.float32, bias=bias.to(DEV), **kw)
+        return
+    y2 = ops.gemm(ad, bd, rg, out_dtype=torch.float32, bias=bias.to(DEV), **kw)
+    f64 = lambda t: t.numpy().astype(np.float64)
+    p0 = O.gemm_acc(a[:, :K0], b[:, :K0], fa, fb) / (f64(sx)[:, None] * f64(sw)[None, :])
+    p1 = O.gemm_acc(a[:, K0:], b[:, K0:], fa, fb) / (f64(sx2)[:, None] * f64(sw2)[None, :])
+    want2 = p0 + p1 + bias.numpy()
+    got2 = y2.cpu().numpy().astype(np.float64)
+    if fa == O.FMT_E4M3:
+        av, bv = np.abs(O.code_values(a, fa)), np.abs(O.code_values(b, fb))
+        slack2 = FP8_ACC_TOL * ((av[:, :K0] @ bv[:, :K0].T) / (f64(sx)[:, None] * f64(sw)[None, :])
+                                + (av[:, K0:] @ bv[:, K0:].T) / (f64(sx2)[:, None] * f64(sw2)[None, :]))
+    else:
+        slack2 = 0.0
+    assert (np.abs(got2 - want2) <= 4e-6 * (np.abs(p0) + np.abs(p1) + np.abs(bias.numpy())[None, :]) + slack2).all()
 
 
 @pytest.mark.parametrize("tile", [0, 11, 15, 16])
