@@ -48,7 +48,7 @@ enum segq_code {
 };
 
 #define SEGQ_MAX_KSEG 8
-#define SEGQ_MAX_RANGES 16
+#define SEGQ_MAX_RANGES 64
 
 int segq_version(void);
 
@@ -189,6 +189,17 @@ typedef struct segq_gemm_desc {
                          * Contents are undefined afterwards.  Replaces nothing in the reference, whose CUTLASS
                          * kernel converts int4 in registers (segquant/src/real_quant/real_gemm.cu:208-305). */
     int64_t workspace_bytes;
+    const float* group_dequant; /* device or NULL.  Group-wise weight scales: entry [g * group_dequant_stride + n]
+                         * is the de-quantisation factor 1 / scale of output column n for contraction columns
+                         * [128 g, 128 g + 128).  When set, the sum of every group is multiplied by its factor
+                         * before it joins the sum of its range (the range's sx and sw still divide the whole):
+                         *   out[m][n] = sum_r ( sum_{g in r} f[g][n] * sum_{k in g} A_r[m][k] B[n][k] )
+                         *                    / (sx_r[m] * sw_r[n]) + bias[n]
+                         * Needs int8 activations, int8 weights or int4 weights with a workspace (above),
+                         * a_sel 0 or 1, every range a whole number of groups, batch == 1, a float out_dtype.
+                         * The reference has per-tensor and per-row weight scales only
+                         * (segquant/src/real_quant/real_gemm.cu:538-638); groups exist here alone. */
+    int64_t group_dequant_stride; /* floats between consecutive groups, >= n */
     segq_krange ranges[SEGQ_MAX_RANGES];
 } segq_gemm_desc;
 

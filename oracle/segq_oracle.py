@@ -291,6 +291,52 @@ def quantize_weights(w, scale_w, fmt: str) -> np.ndarray:
     return codes_of(v, fmt)
 
 
+def group_amax(w, group: int) -> np.ndarray:
+    """|w| maxima over runs of ``group`` input channels: (N, K) -> (N, K / group).
+    Group-wise weight scales are not in the reference (its weight scales are per
+    tensor or per row, segquant/src/real_quant/real_gemm.cu:538-638); a group is
+    defined here as a K segment of the weight with its own per-row scale, so every
+    formula below is the per-row one applied to a (N, group) slice.  Parity
+    unpinned by the reference; pinned by that reduction (tests compare against the
+    per-row functions slice by slice, and ``group == K`` against per-row whole)."""
+    w = _f32(w)
+    n, k = w.shape
+    if k % group:
+        raise ValueError("group must divide K")
+    return np.abs(w).reshape(n, k // group, group).max(axis=-1)
+
+
+def quantize_weights_groups(w, scale_w, group: int, fmt: str) -> np.ndarray:
+    """Weight codes with one multiplicative scale per (row, group): the code rule of
+    ``quantize_weights`` (quantizer.cuh:103-118) with ``scale_w`` of shape
+    (N, K / group).  Returns (N, K) codes (unpacked for int4)."""
+    w = _f32(w)
+    n, k = w.shape
+    s = _f32(scale_w).reshape(n, k // group)
+    v = (w.reshape(n, k // group, group) * s[:, :, None]).astype(np.float32)
+    return codes_of(v.reshape(n, k), fmt)
+
+
+def linear_groups(a_codes, b_codes, scale_x, scale_w, group: int, bias=None) -> np.ndarray:
+    """``out[m, n] = sum_g acc_g[m, n] / (sx[m] * sw[n, g]) + bias[n]`` in fp64, where
+    ``acc_g`` is the exact integer product over group g: the de-quantisation rule of
+    dequantizer.cuh:35-51 applied to every group's partial sum.  ``scale_x`` (M,) or
+    scalar, ``scale_w`` (N, K / group)."""
+    a = np.asarray(a_codes).astype(np.float64)
+    b = np.asarray(b_codes).astype(np.float64)
+    m, k = a.shape
+    n = b.shape[0]
+    sx = np.broadcast_to(np.asarray(scale_x, dtype=np.float64).reshape(-1, 1), (m, 1))
+    sw = np.asarray(scale_w, dtype=np.float64).reshape(n, k // group)
+    out = np.zeros((m, n))
+    for g in range(k // group):
+        acc = a[:, g * group:(g + 1) * group] @ b[:, g * group:(g + 1) * group].T
+        out += acc / (sx * sw[None, :, g])
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.float64).reshape(1, -1)
+    return out
+
+
 # ---------------------------------------------------------------------------
 # contraction (segquant/src/real_quant/real_gemm.cu:208-305)
 # ---------------------------------------------------------------------------

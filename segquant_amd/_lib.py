@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libsegq.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 SEGQ_MAX_KSEG = 8
-SEGQ_MAX_RANGES = 16
+SEGQ_MAX_RANGES = 64
 
 # enum segq_dtype
 F32, F16, BF16, ACC = 0, 1, 2, 3
@@ -54,6 +54,7 @@ class GemmDesc(C.Structure):
         ("batch", C.c_int64), ("batch_stride_a", C.c_int64), ("batch_stride_b", C.c_int64),
         ("batch_stride_out", C.c_int64), ("batch_stride_sx", C.c_int64), ("batch_stride_sw", C.c_int64),
         ("n_ranges", C.c_int32), ("tile", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
+        ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64),
         ("ranges", KRange * SEGQ_MAX_RANGES),
     ]
 

@@ -101,6 +101,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         d->batch_stride_a % 16 || d->batch_stride_b % 16)
         return fail(SEGQ_ERR_ARG, "segq_gemm: a and b need 16-byte aligned bases and row strides");
     if (d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
+    const bool groups = d->group_dequant != nullptr;
+    if (groups) {
+        if (!(i8 || w4) || d->batch != 1 || d->out_dtype == SEGQ_ACC || d->group_dequant_stride < d->n || !al(d->group_dequant, 4))
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need int8 activations, one problem, a float output "
+                                              "and a stride of at least n");
+    }
 
     GemmParams p;
     memset(&p, 0, sizeof(p));
@@ -133,6 +139,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     if (w4 && ktotal > 131071) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: K too large for int4 weights");
     if (kmax > 0x7fffff00) return fail(SEGQ_ERR_ARG, "segq_gemm: K too large");
 
+    if (groups && w4) {
+        const int64_t kp = (kmax + 31) & ~(int64_t)31;
+        if (!d->workspace || !al(d->workspace, 16) || d->workspace_bytes < d->n * kp)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors with int4 weights need %lld bytes of workspace",
+                        (long long)(d->n * kp));
+    }
     if (w4 && d->workspace) {
         // expand b to int8 in the caller's workspace and run the int8 kernels on it
         const int64_t kp = (kmax + 31) & ~(int64_t)31;  // whole 16-byte packed chunks
@@ -179,12 +191,26 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     // several ranges cost a second (fp32) accumulator set, and with it the biggest tiles,
     // unless the accumulators are fp32 already (plain e4m3: rescaled in place)
     const bool fold2 = fold && !(f8 && plain8);
-    if (d->tile == 0) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
+    if (groups) {
+        bool ok = wide_ok && plain8;
+        for (int i = 0; i < d->n_ranges; ++i) ok = ok && d->ranges[i].a_sel < 2;
+        if (!ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need ranges of whole 128-column groups and a_sel 0 or 1");
+        p.grw = d->group_dequant;
+        p.grw_gs = d->group_dequant_stride;
+    }
+    if (d->tile == 0) {
+        if (groups) cfg = FIRST_WIDE_CFG + 3;  // the one tile the group kernel is built for
+        else cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
+    }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
     if (cfg >= FIRST_WIDE_CFG) {
         if (!wide_ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs K ranges in multiples of 128", cfg + 1);
         if (fold2 && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
+        if (groups && cfg != FIRST_WIDE_CFG + 3)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tile %d only", FIRST_WIDE_CFG + 4);
+    } else if (groups) {
+        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tile %d only", FIRST_WIDE_CFG + 4);
     } else if (cfg >= FIRST_BIG_CFG) {
         if (!wide_ok || w4 || fold)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs one range, 8-bit weights and K in multiples of 128", cfg + 1);

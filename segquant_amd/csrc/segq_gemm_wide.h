@@ -431,7 +431,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
 // s_waitcnt immediate for "vmcnt(n) lgkmcnt(0)" on gfx9-family encodings
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }
 
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmParams p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -447,7 +447,19 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // boundary they are rescaled from the finished range's scales to the next
     // one's (acc *= sx' sw' / (sx sw), one fp32 rounding), so the sum stays in
     // units of the current range and the epilogue divides by the last range's.
-    constexpr bool ACCF = FOLD && !F8;
+    //
+    // GRP (int8): every K step of 128 is a group with its own de-quantisation
+    // factor per output column (group-wise weight scales).  The step's int32
+    // sums are multiplied by the factors and added to an fp32 set, which from
+    // there on is treated like e4m3's fp32 accumulators: in units of the current
+    // range, rescaled at range boundaries, scaled by 1/(sx sw) in the epilogue.
+    // The conversion of step s runs between the MFMAs of step s + 1's first
+    // half, each accumulator right before the MFMA that restarts it from zero
+    // (two int32 sets taking turns, so that the conversion spreads over the whole
+    // step, measured no faster: the kernel is held by its one workgroup per CU).
+    static_assert(!GRP || (!F8 && NS == 2), "group factors: int8, two stages");
+    constexpr bool ACCF = FOLD && !F8 && !GRP;
+    constexpr bool HASF = ACCF || GRP;
     const acc_t acc_zero = {0, 0, 0, 0};
 
     static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
@@ -523,17 +535,18 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     };
 
     acc_t acc[TN][TM];
-    v4f accf[ACCF ? TN : 1][ACCF ? TM : 1];
+    v4f accf[HASF ? TN : 1][HASF ? TM : 1];
 #pragma unroll
     for (int a = 0; a < TN; ++a)
 #pragma unroll
         for (int b = 0; b < TM; ++b) acc[a][b] = acc_zero;
-    if constexpr (ACCF) {
+    if constexpr (HASF) {
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
             for (int b = 0; b < TM; ++b) accf[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
     }
+
 
     const int f_sw = swz(lrow);
     const int a_frag = (wm * WM + lrow) * BK;
@@ -571,8 +584,23 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     };
     const int m_base = m0 + wm * WM + lrow;
     const int n_base = n0 + wn * WN + 4 * lgrp;
-    auto fold = [&](int r) {
-        if constexpr (FOLD && F8) {
+    // the group factors of the step in ring slot `slot` times this step's sums, into the fp32 set
+    auto add_groups = [&](auto& set, const float* grw, int slot) __attribute__((always_inline)) {
+        if constexpr (GRP) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                const v4f g = *reinterpret_cast<const v4f*>(grw + slot * BN + wn * WN + a * 16 + 4 * lgrp);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    accf[a][b] += __builtin_convertvector(set[a][b], v4f) * g;
+                    set[a][b] = acc_zero;
+                }
+            }
+        }
+    };
+    auto fold = [&](int r) __attribute__((always_inline)) {
+        if constexpr (FOLD && (F8 || GRP)) {
+            auto& facc = [&]() -> auto& { if constexpr (GRP) return accf; else return acc; }();
             if (r + 1 < p.nr) {  // rescale to the next range's units
                 const float* sx = p.r[r].sx + z * p.bsSx;
                 const float* sw = p.r[r].sw + z * p.bsSw;
@@ -594,7 +622,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                         fw[v] = sw2[n * cs2] * __builtin_amdgcn_rcpf(sw[n * cs]);
                     }
 #pragma unroll
-                    for (int b = 0; b < TM; ++b) acc[a][b] = acc[a][b] * (fw * fx[b]);
+                    for (int b = 0; b < TM; ++b) facc[a][b] = facc[a][b] * (fw * fx[b]);
                 }
             }
         }
@@ -645,6 +673,21 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // trip to memory, and without the ~70 small loads per wave it would take there.
     constexpr int EPI_FLOATS = BM + 2 * BN, EPI_IT = (EPI_FLOATS + NT - 1) / NT;
     float* const epi = reinterpret_cast<float*>(smem + NS * (BM + BN) * BK);
+    // group factors: a ring of four rows of BN floats behind the epilogue's vectors.  The row of
+    // step s arrives with the step's operands and is read all through step s + 1, at whose end
+    // the row of step s + 3 is already on its way: it must not land in the same slot
+    float* const grw = epi + EPI_FLOATS;
+    int lslot = 0, cslot = 0, pslot = 0;  // slots of the step being loaded / multiplied / converted
+    auto dma_g = [&]() {
+        if constexpr (GRP) {
+            if (wave < BN / 64) {
+                const int n = min(n0 + wave * 64 + lane, p.N - 1);
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.grw + (int64_t)(lk >> 7) * p.grw_gs + n),
+                                                 (lds_ptr_t)(grw + lslot * BN + wave * 64), 4, 0, 0);
+            }
+            lslot = (lslot + 1) & 3;
+        }
+    };
     const int r_epi = ACCF ? 0 : p.nr - 1;  // the range whose units the accumulators end up in
     float epi_val[EPI_IT];
     const bool want_epi = p.out_dtype != SEGQ_ACC;  // raw accumulators come with no scales at all (null pointers)
@@ -669,12 +712,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (int t = 0; t < NS; ++t) {
         if (t < steps) {
             dma(la + lk, Bb + lk, t);
+            dma_g();
             advance_load();
             ++issued;
         }
     }
-    if (issued == NS) wait_dma(std::integral_constant<int, NS - 1>{});
-    else wait_dma(std::integral_constant<int, 0>{});
+    if (issued == NS && !GRP) wait_dma(std::integral_constant<int, NS - 1>{});
+    else wait_dma(std::integral_constant<int, 0>{});  // (with group factors the waves' DMA counts differ)
 #pragma unroll
     for (int i = 0; i < EPI_IT; ++i) {
         const int e = i * NT + tid;
@@ -760,17 +804,33 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
         buf = nbuf;
     };
-    auto step_i8 = [&](auto dma_c, auto more_c) {
+    auto step_i8 = [&](auto dma_c, auto more_c) __attribute__((always_inline)) {
         constexpr bool DMA_ = decltype(dma_c)::value;
         constexpr bool MORE_ = decltype(more_c)::value;
         const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
+        // group schedule: the previous step's factors, one column block ahead of their use
+        // (the first step adds zeros)
+        const float* const gsrc = grw + pslot * BN + wn * WN + 4 * lgrp;
+        v4f gv = {0.f, 0.f, 0.f, 0.f}, gnext = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (GRP) gnext = *reinterpret_cast<const v4f*>(gsrc);
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
                 const int i = a * TM + b;
+                if constexpr (GRP) {
+                    if (b == 0) {
+                        gv = gnext;
+                        if (a + 1 < TN) gnext = *reinterpret_cast<const v4f*>(gsrc + (a + 1) * 16);
+                    }
+                }
                 if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(buf, 1, i / RD_EVERY);
-                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
+                if constexpr (GRP) {
+                    accf[a][b] += __builtin_convertvector(acc[a][b], v4f) * gv;
+                    acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc_zero, 0, 0, 0);
+                } else {
+                    acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
@@ -788,6 +848,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 const int i = a * TM + b;
                 if constexpr (DMA_) {
                     if (i % DM_EVERY == DM_EVERY - 1 && i / DM_EVERY < NDM) dma1(ap, bp, buf, i / DM_EVERY);
+                    if (i == NMF - 1) dma_g();
                 }
                 if constexpr (MORE_) {
                     if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(nbuf, 0, i / RD_EVERY);
@@ -802,7 +863,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0), vmcnt untouched
         if constexpr (DMA_) advance_load();
         ck += BK;
+        pslot = cslot;
+        cslot = (cslot + 1) & 3;
         if (ck >= ck1) {  // the range is complete: fold it, move to the next one
+            if constexpr (GRP && FOLD) add_groups(acc, grw, pslot);  // this step's sums are still in the old range's units
             if constexpr (FOLD) fold(cr);
             ++cr;
             const int rr = min(cr, p.nr - 1);
@@ -811,7 +875,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
         buf = nbuf;
     };
-    auto step = [&](auto dma_c, auto more_c) {
+    auto step = [&](auto dma_c, auto more_c) __attribute__((always_inline)) {
         if constexpr (F8) step8(dma_c, more_c);
         else step_i8(dma_c, more_c);
     };
@@ -819,7 +883,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
     for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
     if (s < steps) step(std::false_type{}, std::false_type{});
-    wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, r_epi, epi);
+    if constexpr (GRP) {
+        add_groups(acc, grw, pslot);  // the last step's sums
+        v4f none[1][1];
+        wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, false>(p, accf, none, smem, z, m0, n0, wave, lane, r_epi, epi);
+    } else {
+        wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, r_epi, epi);
+    }
 }
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool ASEL>
@@ -838,10 +908,11 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 }
 
 // wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false>
 int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
-    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS>;
-    constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4;  // the stages and the epilogue's vectors
+    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP>;
+    // the stages, the epilogue's vectors, and the ring of group factors
+    constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4 + (GRP ? 4 * BN * 4 : 0);
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
@@ -855,6 +926,17 @@ int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 
 template <int FMT, bool B4>
 int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st) {
+    if constexpr (!B4 && FMT == GEMM_I8) {
+        if (p.grw) {  // group-wise factors (the host has checked: plain codes, K ranges in whole steps)
+            if (asel) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need plain codes");
+            // one tile only: with a second accumulator set, the factors and the conversion's
+            // temporaries the 64 x 64 wave tiles of 256 x 128 and 128 x 256 spill ~100 registers
+            if (wcfg == 3)
+                return fold ? launch_pipe_instance<128, 128, 2, 4, FMT, true, 2, true>(p, batch, st)
+                            : launch_pipe_instance<128, 128, 2, 4, FMT, false, 2, true>(p, batch, st);
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on the 128x128 tile of eight waves");
+        }
+    }
     if constexpr (!B4) {
         constexpr bool F8W = FMT == GEMM_F8;  // the e4m3 schedule wants three or more column blocks per wave
         if (!asel) {  // plain 8-bit operands, both straight to LDS: the software-pipelined kernel

@@ -175,7 +175,8 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
          out_dtype, lda: int, ldb: int, a_neg: Optional[torch.Tensor] = None,
          bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
-         tile: int = 0, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+         tile: int = 0, workspace: Optional[torch.Tensor] = None,
+         group_dequant: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
@@ -209,6 +210,11 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
     if workspace is not None:
         _need_cuda(workspace)
         d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()
+    if group_dequant is not None:
+        _need_cuda(group_dequant)
+        if group_dequant.dtype != torch.float32 or group_dequant.dim() != 2 or group_dequant.stride(1) != 1:
+            raise RuntimeError("group_dequant is a float32 matrix (groups, n) with contiguous rows")
+        d.group_dequant = group_dequant.data_ptr(); d.group_dequant_stride = group_dequant.stride(0)
     for i, r in enumerate(ranges):
         kr = d.ranges[i]
         kr.k_begin = r.k_begin; kr.k_len = r.k_len; kr.a_sel = r.a_sel
@@ -344,6 +350,37 @@ def real_quantized_quantize_weights(fmt: str, weights: torch.Tensor, outputs: to
     else:  # the float overload is noconvert (seg_utils.h:99)
         raise TypeError("scale_w must be a python float or a float32 tensor")
     L.check(rc)
+
+
+def quantize_weights_groups(fmt: str, weights: torch.Tensor, scales: torch.Tensor, group: int = 128) -> torch.Tensor:
+    """Weight codes with one scale per (row, group of ``group`` contraction columns).
+
+    ``weights`` is (n, k) float, ``scales`` a contiguous float32 (k / group, n) matrix of
+    multiplicative scales (``code = round(w * scale)``), the layout whose reciprocal
+    ``segq_gemm`` takes as ``group_dequant``.  Returns (n, k) codes, or (n, k / 2) bytes
+    for int4.  The reference has no group-wise scales
+    (segquant/src/real_quant/real_gemm.cu:538-638 takes a scalar or one scale per row);
+    a group is quantised exactly like a K segment with static per-row scales, so this
+    runs on ``segq_quantize`` in slices of at most SEGQ_MAX_KSEG groups.
+    """
+    _need_cuda(weights, scales)
+    if weights.dim() != 2 or not weights.is_contiguous():
+        raise RuntimeError("tensor must be contiguous")
+    n, k = weights.shape
+    if group % 32 or k % group:
+        raise RuntimeError("the group size must be a multiple of 32 that divides k")
+    ng = k // group
+    if scales.dtype != torch.float32 or tuple(scales.shape) != (ng, n) or not scales.is_contiguous():
+        raise RuntimeError(f"scales must be a contiguous float32 ({ng}, {n}) matrix")
+    out = torch.empty((n, k // 2 if fmt == FMT_INT4 else k), dtype=code_dtype(fmt), device=weights.device)
+    step = L.SEGQ_MAX_KSEG
+    for g0 in range(0, ng, step):
+        g1 = min(ng, g0 + step)
+        c0, c1 = g0 * group, g1 * group
+        oc0, oc1 = (c0 // 2, c1 // 2) if fmt == FMT_INT4 else (c0, c1)
+        quantize(weights[:, c0:c1], fmt, scales[g0:], row_stride=1,
+                 kseg_bounds=[i * group for i in range(g1 - g0 + 1)], kseg_stride=n, out=out[:, oc0:oc1])
+    return out
 
 
 def fake_e4m3fy(inputs: torch.Tensor) -> torch.Tensor:

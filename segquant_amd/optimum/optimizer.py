@@ -81,6 +81,9 @@ class BaseOptimizer:
 
     def call_func(self, batch_input: torch.Tensor, batch_weight: torch.Tensor):
         if self.real_quant:
+            if getattr(self.weight_calibrators[0], "group_size", None) is not None:
+                # the reference's operators take one weight scale per segment or per row
+                raise NotImplementedError("group-wise weight scales run on the fused route only (chunked=False)")
             if self.input_calibrators[0].dynamic:
                 # The reference calls a method that does not exist here
                 # (optimizer.py:96-100).  Recalibrate each segment on this
@@ -218,6 +221,21 @@ class DefaultOptimizer(BaseOptimizer):
         wcodes = wm.weight_tensor
         wcodes = wcodes.reshape(N, K // 2 if fw == ops.FMT_INT4 else K).contiguous()
         dev = wm.device()
+        group = getattr(self.weight_calibrators[0], "group_size", None)
+        if group is not None:
+            # group-wise weight scales (rows, K / group): the kernel takes their reciprocals as a
+            # (K / group, N) matrix of factors; the per-column scale it also applies is 1
+            if group != 128:
+                raise NotImplementedError("the kernel path has group-wise weight scales for groups of 128")
+            per_row = torch.cat([_as_f32(c.scale, dev).reshape(-1, K // group) for c in self.weight_calibrators])
+            bounds = [0, K]
+            if self.seg_mode != "weight":
+                bounds = [0]
+                for c in self.chunksizes:
+                    bounds.append(bounds[-1] + c)
+            self._plan = dict(fa=fa, fw=fw, w=wcodes, sw=torch.ones(1, dtype=torch.float32, device=device), sw_cs=0,
+                              bounds=bounds, N=N, K=K, group_dequant=(1.0 / per_row).t().contiguous().to(device))
+            return self._plan
         wscales = [_as_f32(c.scale, dev).reshape(-1) for c in self.weight_calibrators]
         if self.seg_mode == "weight":
             # per-segment or per-channel -> one scale per output column (or a single scalar)
@@ -292,7 +310,9 @@ class DefaultOptimizer(BaseOptimizer):
         # library N x K bytes to expand the weights into once per launch (the int8 kernels
         # then run); with few tokens reading half the weight bytes matters more
         # (measured, K 1280, N 10240: 161 -> 119 us at 8192 tokens, no gain at 2048)
-        ws = ops.int4_workspace(x.device, N * K) if plan["fw"] == ops.FMT_INT4 and M >= 3072 else None
+        # (group-wise scales run on the int8 kernels only: always lend)
+        gdq = plan.get("group_dequant")
+        ws = ops.int4_workspace(x.device, N * K) if plan["fw"] == ops.FMT_INT4 and (M >= 3072 or gdq is not None) else None
         out = ops.gemm(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
-                       lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws)
+                       lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws, group_dequant=gdq)
         return out.view(*x.shape[:-1], N)

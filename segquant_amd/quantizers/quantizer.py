@@ -30,7 +30,13 @@ def _bcast(x: torch.Tensor, s, axis):
 
 
 class BaseQuantizer:
-    def __init__(self, axis=None, dual_scale=False, real_quant=False, dynamic=False, dummy=False):
+    def __init__(self, axis=None, dual_scale=False, real_quant=False, dynamic=False, dummy=False, group_size=None):
+        # group_size: weights only, with axis=1 -- one scale per (row, run of group_size
+        # input channels) instead of one per row.  Not in the reference (its weight scales
+        # are per tensor or per row); the scale has shape (rows, in_features / group_size).
+        self.group_size = group_size
+        if group_size is not None and (axis != 1 or dual_scale or dynamic):
+            raise AssertionError("group_size is for static weight scales on axis 1")
         self.axis = axis
         self.dual_scale = dual_scale
         self.real_quant = real_quant
@@ -85,9 +91,17 @@ class BaseQuantizer:
             self.neg_scale = self._ratio(self.neg_limit, self._track("neg_amax", nmax))
             self.pos_scale = self._ratio(self.pos_limit, self._track("pos_amax", pmax))
         else:
-            a = x.abs().max().item() if self.axis is None else x.abs().amax(dim=self.axis)
+            if self.group_size is not None:
+                a = self._grouped(x).abs().amax(dim=-1)
+            else:
+                a = x.abs().max().item() if self.axis is None else x.abs().amax(dim=self.axis)
             self.scale = self._ratio(self.pos_limit, self._track("amax", a))
         self.zero_point = 0
+
+    def _grouped(self, x: torch.Tensor) -> torch.Tensor:
+        if x.dim() != 2 or x.shape[1] % self.group_size:
+            raise ValueError(f"group_size {self.group_size} needs a 2-D weight whose columns it divides")
+        return x.reshape(x.shape[0], x.shape[1] // self.group_size, self.group_size)
 
     def calibrate(self, x: torch.Tensor):
         if self.dummy:
@@ -112,6 +126,12 @@ class BaseQuantizer:
         if self.real_quant:
             assert not self.dual_scale, "Weight quantization does not support dual scale."
             ext = self._weight_ext()
+            if ext is not None and self.group_size is not None:
+                g = x.shape[1] // self.group_size
+                if not isinstance(self.scale, torch.Tensor) or tuple(self.scale.shape) != (x.shape[0], g):
+                    raise ValueError(f"group-wise weight scale must have shape ({x.shape[0]}, {g})")
+                scales = self.scale.to(dtype=torch.float32, device=x.device).t().contiguous()
+                return ext.quantize_weights_groups(x.contiguous(), scales, self.group_size)
             if ext is not None:
                 res = ext.create_quantized_weights(x)
                 if self.axis is None:
@@ -133,7 +153,7 @@ class BaseQuantizer:
 
 class IntQuantizer(BaseQuantizer):
     def __init__(self, num_bits=8, symmetric=True, axis=None, dual_scale=False, real_quant=False, dynamic=False,
-                 dummy=False):
+                 dummy=False, group_size=None):
         self.num_bits = num_bits
         self.symmetric = symmetric
         self.qmin = -(2 ** (num_bits - 1))
@@ -141,7 +161,9 @@ class IntQuantizer(BaseQuantizer):
         # the negative side has one more code than the positive one
         self.pos_limit = float(self.qmax)
         self.neg_limit = float(-self.qmin)
-        super().__init__(axis, dual_scale, real_quant, dynamic, dummy)
+        if group_size is not None and not symmetric:
+            raise AssertionError("group_size is for symmetric weights")
+        super().__init__(axis, dual_scale, real_quant, dynamic, dummy, group_size)
 
     def calibrate(self, x: torch.Tensor):
         if self.dummy or self.symmetric:
@@ -167,6 +189,10 @@ class IntQuantizer(BaseQuantizer):
             q = torch.where(nonneg, torch.clamp(torch.round(x * ps), 0, self.qmax),
                             torch.clamp(torch.round(x * ns), self.qmin, 0))
             return torch.where(nonneg, q / ps, q / ns).to(x.dtype)
+        if self.group_size is not None:
+            xg, sg = self._grouped(x), self.scale.unsqueeze(-1)
+            q = torch.clamp(torch.round(xg * sg), self.qmin, self.qmax)
+            return (q / sg).reshape(x.shape).to(x.dtype)
         s = _bcast(x, self.scale, self.axis)
         zp = _bcast(x, self.zero_point, self.axis)
         q = torch.clamp(torch.round(x * s) + zp, self.qmin, self.qmax)
@@ -191,7 +217,9 @@ class IntQuantizer(BaseQuantizer):
 
 class FloatQuantizer(BaseQuantizer):
     def __init__(self, exp_bits=4, mant_bits=3, axis=None, dual_scale=False, real_quant=False, dynamic=False,
-                 dummy=False):
+                 dummy=False, group_size=None):
+        if group_size is not None:
+            raise AssertionError("group_size is for integer weights")
         self.exp_bits = exp_bits
         self.mant_bits = mant_bits
         if (exp_bits, mant_bits) == (4, 3):

@@ -85,6 +85,12 @@ class RealQuantExt:
             raise RuntimeError(f"{self.name} has no single weight format")
         ops.real_quantized_quantize_weights(self.weight_fmt, weights, outputs, scale_w)
 
+    def quantize_weights_groups(self, weights, scales, group):
+        """Codes for group-wise scales ((k / group, n) float32); not in the reference."""
+        if self.weight_fmt is None:
+            raise RuntimeError(f"{self.name} has no single weight format")
+        return ops.quantize_weights_groups(self.weight_fmt, weights, scales, group)
+
 
 def _load(name, prefixes, weight_fmt, verbose, required):
     if name in _loaded_extensions:

@@ -34,6 +34,7 @@ class LinearSpec:
     act_axis: Optional[int] = None           # None per tensor, -1 per token
     dynamic: bool = False
     weight_axis: Optional[int] = None        # None per tensor / per segment, 1 per channel
+    weight_group: Optional[int] = None       # with weight_axis 1: one scale per run of this many input channels
     dual_segments: List[int] = field(default_factory=list)  # K segments (or [0]) that use DualScale
     outlier: str = "x20"                     # x20 | x30 | student_t
     gelu_segments: List[int] = field(default_factory=list)  # segments passed through gelu_tanh
@@ -115,7 +116,7 @@ def config_linears(config: int, M: Optional[int] = None) -> List[LinearSpec]:
         ]
     if config == 4:
         m = M or 8192
-        kw = dict(weight="int4", act_axis=-1, dynamic=True, weight_axis=1, outlier="x20")
+        kw = dict(weight="int4", act_axis=-1, dynamic=True, weight_axis=1, weight_group=128, outlier="x20")
         return [
             LinearSpec("geglu_proj", 4, m, 1280, 10240, chunksizes=[5120] * 2, tensor_index=0, **kw),
             LinearSpec("ff_out", 4, m, 5120, 1280, tensor_index=1, **kw),
@@ -150,7 +151,8 @@ def build_layer(spec: LinearSpec, device="cuda:0", real_quant=True, x: Optional[
         custom_weight_tensor=w, custom_bias_tensor=b, input_quant_type=spec.act, weight_quant_type=spec.weight,
         input_quant_args={"real_quant": real_quant, "dual_scale": dual, "axis": spec.act_axis,
                           "dynamic": spec.dynamic},
-        weight_quant_args={"real_quant": real_quant, "axis": spec.weight_axis}, device=device)
+        weight_quant_args={"real_quant": real_quant, "axis": spec.weight_axis,
+                           **({"group_size": spec.weight_group} if spec.weight_group else {})}, device=device)
     layer.calibrate(x.to(device))
     layer.finish_calibrate()
     return layer, x

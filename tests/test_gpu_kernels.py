@@ -352,6 +352,57 @@ def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
     assert (y0 - y1).abs().max().item() <= 2e-6 * y0.abs().max().item()
 
 
+@pytest.mark.parametrize("fmt_w", [O.FMT_INT4, O.FMT_INT8])
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_group_wise_weight_scales(ops, fmt_w, dt):
+    """Weights with one scale per (row, group of 128 input channels): codes bit-exact against
+    the oracle, and the GEMM with group factors against the closed form, on ragged M and N,
+    on a single range with per-token scales, and on K segments with a two-tensor DualScale
+    segment.  (No counterpart in the reference: the oracle's group functions are the per-row
+    ones applied group by group.)"""
+    M, N, K, G = 203, 330, 1280, 128
+    g = torch.Generator().manual_seed(31)
+    w = torch.randn(N, K, generator=g) * 0.02
+    w[:, 5] *= 30  # one group per row with a far larger maximum than its neighbours
+    bits = 4 if fmt_w == O.FMT_INT4 else 8
+    sw = O.int_scale(O.group_amax(w.numpy(), G), bits)  # (N, K / G)
+    sw_t = torch.from_numpy(np.ascontiguousarray(sw.T)).to(DEV)
+    codes = ops.quantize_weights_groups(fmt_w, w.to(DEV), sw_t, G)
+    want_codes = O.quantize_weights_groups(w.numpy(), sw, G, fmt_w)
+    assert np.array_equal(_codes_np(codes, fmt_w), want_codes)
+    a = _rand_codes((M, K), O.FMT_INT8, 32)
+    a2 = _rand_codes((M, K), O.FMT_INT8, 33)
+    ad, a2d = _to_dev_codes(a, O.FMT_INT8), _to_dev_codes(a2, O.FMT_INT8)
+    sx = (torch.rand(M, generator=g) + 0.5)
+    sx2 = (torch.rand(M, generator=g) + 0.5)
+    bias = torch.randn(N, generator=g)
+    one = torch.ones(1, device=DEV)
+    factors = (1.0 / sw_t).contiguous()
+    ws = torch.empty(N * K, dtype=torch.uint8, device=DEV)
+    kw = dict(m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=fmt_w, out_dtype=TDT[dt], lda=K, ldb=K // 2 if fmt_w == O.FMT_INT4 else K,
+              bias=bias.to(DEV), workspace=ws, group_dequant=factors)
+    tol = 4e-6 if dt == "fp32" else 2.0 ** -8
+    # (a) one range, per-token scales
+    out = ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 0, 1, 0)], **kw)
+    want = O.linear_groups(a, want_codes, sx.numpy(), sw, G, bias.numpy())
+    assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max()
+    # (b) K segments [0, 512) and [512, 1280); the second read twice, from two code tensors
+    rg = [ops.Range(0, 512, sx.to(DEV), one, 0, 1, 0), ops.Range(512, K - 512, sx2.to(DEV), one, 0, 1, 0),
+          ops.Range(512, K - 512, sx.to(DEV), one, 1, 1, 0)]
+    out = ops.gemm(ad, codes, rg, a_neg=a2d, **kw)
+    nog = O.linear_groups  # per part: groups are indexed by absolute K, so slice the scales with the codes
+    want = (nog(a[:, :512], want_codes[:, :512], sx.numpy(), sw[:, :4], G) +
+            nog(a[:, 512:], want_codes[:, 512:], sx2.numpy(), sw[:, 4:], G) +
+            nog(a2[:, 512:], want_codes[:, 512:], sx.numpy(), sw[:, 4:], G) + bias.numpy().astype(np.float64))
+    assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max()
+    # what the group kernel does not serve is refused, not approximated
+    with pytest.raises(RuntimeError):
+        ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 2, 1, 0)], **kw)
+    if fmt_w == O.FMT_INT4:
+        with pytest.raises(RuntimeError):
+            ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 0, 1, 0)], **dict(kw, workspace=None))
+
+
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
 def test_gemm_sign_selected_halves_of_merged_codes(ops, fmt):
     M, N, K = 70, 90, 320

@@ -44,16 +44,32 @@ def oracle_layer_output(layer, spec, x_np, out_dtype):
     M = x_np.shape[0]
     bounds = segment_bounds(spec)
     single, dualf = _scale_fn(fa)
-    # weight scale per output column
+    # weight scale per output column, or per (column, group of input channels)
     wcals = opt.weight_calibrators
-    if spec.seg_mode == "weight" and len(wcals) > 1:
+    group = getattr(wcals[0], "group_size", None)
+    if group:
+        sw_groups = np.concatenate([_np32(c.scale).reshape(-1, K // group) for c in wcals]).astype(np.float32)
+        sw = None
+    elif spec.seg_mode == "weight" and len(wcals) > 1:
         sw = np.concatenate([np.broadcast_to(np.float32(_np32(torch.as_tensor(c.scale))).reshape(-1), (n,)) if
                              np.ndim(c.scale) == 0 or torch.as_tensor(c.scale).numel() == 1 else
                              _np32(c.scale) for c, n in zip(wcals, opt.chunksizes)])
     else:
         s0 = torch.as_tensor(wcals[0].scale).float().cpu().numpy().reshape(-1)
         sw = np.broadcast_to(s0, (N,)) if s0.size == 1 else s0
-    sw = sw.astype(np.float32).reshape(1, N)
+    if sw is not None:
+        sw = sw.astype(np.float32).reshape(1, N)
+
+    def dequantised(codes, k0, k1, sx):
+        """sum over the weight-scale blocks of [k0, k1) of acc / (sx * sw)"""
+        if not group:
+            return O.gemm_acc(codes, wq[:, k0:k1], fa, fw) / (sx.astype(np.float64) * sw)
+        t = np.zeros((M, N), dtype=np.float64)
+        for g0 in range(k0, k1, group):
+            swg = sw_groups[:, g0 // group].reshape(1, N)
+            t += O.gemm_acc(codes[:, g0 - k0:g0 - k0 + group], wq[:, g0:g0 + group], fa, fw) / (sx.astype(np.float64) * swg)
+        return t
+
     y = np.zeros((M, N), dtype=np.float64)
     for s in range(len(bounds) - 1):
         k0, k1 = bounds[s], bounds[s + 1]
@@ -79,11 +95,11 @@ def oracle_layer_output(layer, spec, x_np, out_dtype):
             ns = np.float32(ns).reshape(-1)
             nsb = ns.reshape(-1, 1) if ns.size > 1 else ns.reshape(1, 1)
             cp, cn = O.quantize_act_dual(xs[None], ps if ps.size > 1 else ps[:1], ns if ns.size > 1 else ns[:1], fa)
-            y += O.gemm_acc(cp[0], wq[:, k0:k1], fa, fw) / (psb.astype(np.float64) * sw)
-            y += O.gemm_acc(cn[0], wq[:, k0:k1], fa, fw) / (nsb.astype(np.float64) * sw)
+            y += dequantised(cp[0], k0, k1, psb)
+            y += dequantised(cn[0], k0, k1, nsb)
         else:
             c = O.quantize_act(xs[None], ps if ps.size > 1 else ps[:1], fa)
-            y += O.gemm_acc(c[0], wq[:, k0:k1], fa, fw) / (psb.astype(np.float64) * sw)
+            y += dequantised(c[0], k0, k1, psb)
     if layer.bias:
         y += _np32(layer.bias_data).astype(np.float64)
     return y

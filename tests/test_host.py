@@ -127,6 +127,28 @@ def test_int_quantizer_scales_and_fake_quant(bits):
     assert (qz.pos_scale, qz.neg_scale) == (1.0, 1.0)
 
 
+def test_int_quantizer_group_scales_and_fake_quant():
+    """group_size: one weight scale per (row, run of input channels); the oracle's group
+    functions are the checker."""
+    from segquant_amd.quantizers.quantizer import FloatQuantizer, IntQuantizer
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(10, 96, generator=g) * 0.05
+    q = IntQuantizer(num_bits=4, axis=1, group_size=32)
+    q.calibrate(w)
+    want = O.int_scale(O.group_amax(w.numpy(), 32), 4)
+    assert tuple(q.scale.shape) == (10, 3) and np.array_equal(q.scale.numpy(), want)
+    codes = O.quantize_weights_groups(w.numpy(), want, 32, O.FMT_INT4).astype(np.float32)
+    deq = (codes.reshape(10, 3, 32) / want[:, :, None]).reshape(10, 96)
+    assert np.array_equal(q.fake_quantize(w).numpy(), deq)
+    for bad in (dict(axis=None), dict(axis=1, dual_scale=True), dict(axis=1, dynamic=True), dict(axis=1, symmetric=False)):
+        with pytest.raises(AssertionError):
+            IntQuantizer(num_bits=4, group_size=32, **bad)
+    with pytest.raises(AssertionError):
+        FloatQuantizer(axis=1, group_size=32)
+    with pytest.raises(ValueError):
+        IntQuantizer(num_bits=4, axis=1, group_size=40).calibrate(w)
+
+
 def test_float_quantizer_scales_and_fake_quant():
     from segquant_amd.quantizers.quantizer import FloatQuantizer, QuantizerRegistry
     g = torch.Generator().manual_seed(1)

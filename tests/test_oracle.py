@@ -292,3 +292,52 @@ def test_round_to_bf16_matches_torch():
     g = torch.Generator().manual_seed(1)
     x = torch.randn(100000, generator=g) * 100
     assert np.array_equal(O.round_to_bf16(x.numpy()), x.to(torch.bfloat16).float().numpy())
+
+
+# ---- group-wise weight scales (exist in this build only) ----------------------
+def test_group_functions_reduce_to_the_per_row_ones():
+    """A group is a K slice of the weight with per-row scales: slice by slice the
+    group functions must equal the per-row functions, and one group spanning all
+    of K must equal the per-row result on the whole matrix."""
+    rng = np.random.default_rng(11)
+    n, k, g = 12, 96, 32
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    amax = O.group_amax(w, g)
+    assert amax.shape == (n, k // g)
+    for j in range(k // g):
+        np.testing.assert_array_equal(amax[:, j], np.abs(w[:, j * g:(j + 1) * g]).max(axis=1))
+    scale = O.int_scale(amax, bits=4)
+    codes = O.quantize_weights_groups(w, scale, g, O.FMT_INT4)
+    for j in range(k // g):
+        np.testing.assert_array_equal(codes[:, j * g:(j + 1) * g],
+                                      O.quantize_weights(w[:, j * g:(j + 1) * g], scale[:, j], O.FMT_INT4))
+    whole = O.int_scale(O.group_amax(w, k), bits=4)
+    np.testing.assert_array_equal(O.quantize_weights_groups(w, whole, k, O.FMT_INT4),
+                                  O.quantize_weights(w, whole.reshape(-1), O.FMT_INT4))
+    # every group reaches the end of the code range at its own maximum
+    assert (np.abs(codes).reshape(n, k // g, g).max(axis=-1) == 7).all()
+
+
+def test_linear_groups_against_bruteforce_and_per_row():
+    rng = np.random.default_rng(12)
+    m, n, k, g = 5, 7, 64, 16
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    sx = (rng.random(m) + 0.5).astype(np.float32)
+    sw = (rng.random((n, k // g)) + 0.5).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    got = O.linear_groups(a, b, sx, sw, g, bias)
+    want = np.zeros((m, n))
+    for i in range(m):
+        for j in range(n):
+            t = 0.0
+            for kk in range(k):
+                t += int(a[i, kk]) * int(b[j, kk]) / (float(sx[i]) * float(sw[j, kk // g]))
+            want[i, j] = t + float(bias[j])
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-9)
+    # equal scales in all groups of a row: the per-row de-quantisation of the whole sum
+    sw_same = np.repeat(sw[:, :1], k // g, axis=1)
+    acc = O.gemm_acc(a, b, O.FMT_INT8, O.FMT_INT4)
+    np.testing.assert_allclose(O.linear_groups(a, b, sx, sw_same, g),
+                               acc / (sx.astype(np.float64)[:, None] * sw_same[:, 0].astype(np.float64)[None, :]),
+                               rtol=1e-12)
