@@ -87,7 +87,23 @@ const char* segq_last_error(void);
  * dual: :183-203; e4m3: 448) and quantises with it.  Needs row_stride == 1 or a
  * single row per scale; has no counterpart kernel in the reference, whose
  * dynamic mode calls a method that does not exist (optimum/optimizer.py:96-100).
+ *
+ * pre_op != SEGQ_PRE_NONE fuses the activation function of the layer in front:
+ * what is quantised (and, when dynamic, what the maximum is taken of) is op(x),
+ * or x * op(gate) when gate is given, each operator's result rounded to x_dtype
+ * as that layer would have stored it.  These are the reference's GELU(tanh) MLP
+ * (backend/torch/modules/transformer_flux.py:91), GELU / SiLU
+ * (backend/torch/layers/activations.py:52-57) and the gated GEGLU / SwiGLU
+ * (activations.py:77-80, :110-121), which there run as separate torch operators
+ * writing a full-size tensor that the quantise kernel then reads back.
  * ---------------------------------------------------------------------- */
+typedef enum segq_pre_op {
+    SEGQ_PRE_NONE = 0,
+    SEGQ_PRE_GELU_TANH = 1, /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) */
+    SEGQ_PRE_GELU = 2,      /* 0.5 x (1 + erf(x / sqrt(2))) */
+    SEGQ_PRE_SILU = 3       /* x / (1 + exp(-x)) */
+} segq_pre_op;
+
 typedef struct segq_quant_desc {
     const void* x;      /* device, rows x cols, x_dtype, row stride ldx elements */
     int32_t x_dtype;    /* segq_dtype: F32 | F16 | BF16 */
@@ -109,6 +125,9 @@ typedef struct segq_quant_desc {
     uint32_t dual_kseg_mask;
     int32_t dynamic;
     int64_t kseg_bounds[SEGQ_MAX_KSEG + 1]; /* column segment i = [bounds[i], bounds[i+1]); multiples of 16 */
+    int32_t pre_op;     /* segq_pre_op */
+    const void* gate;   /* device or NULL: rows x cols of x_dtype, row stride ld_gate; needs a pre_op */
+    int64_t ld_gate;
 } segq_quant_desc;
 
 int segq_quantize(const segq_quant_desc* d, segq_stream_t stream);

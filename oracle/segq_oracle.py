@@ -291,6 +291,40 @@ def quantize_weights(w, scale_w, fmt: str) -> np.ndarray:
     return codes_of(v, fmt)
 
 
+def activation(x, op: str, gate=None, dtype: str = "fp32") -> np.ndarray:
+    """The activation function in front of a linear, as torch evaluates it for a
+    tensor of ``dtype``: in fp32, each operator's result rounded to ``dtype``
+    (backend/torch/layers/activations.py:52-57 GELU, :77-80 SwiGLU, :110-121
+    GEGLU; backend/torch/modules/transformer_flux.py:91 GELU(tanh)).  ``op`` is
+    "gelu_tanh", "gelu" or "silu"; with ``gate`` the result is x * op(gate).
+    The arithmetic around the transcendental function is done in fp32 step by
+    step, as torch and the kernel do it (so 1 + tanh(.) cancels to exactly 0 in
+    the far negative tail, as it does there); tanh / erf / exp themselves are
+    taken in fp64 and rounded to fp32, i.e. correctly rounded, where a device's
+    tanhf / erff / expf may be an ulp off.  Pinned against torch's CPU operators
+    (library routine) in the tests."""
+    from scipy.special import erf
+    f32 = np.float32
+
+    def f(t):
+        t = _f32(t)
+        if op == "gelu_tanh":
+            inner = f32(0.7978845608028654) * (t + f32(0.044715) * (t * t * t))
+            r = f32(0.5) * t * (f32(1.0) + np.tanh(inner.astype(np.float64)).astype(f32))
+        elif op == "gelu":
+            r = t * f32(0.5) * (f32(1.0) + erf((t * f32(0.7071067811865476)).astype(np.float64)).astype(f32))
+        elif op == "silu":
+            with np.errstate(over="ignore"):
+                r = t / (f32(1.0) + np.exp(-t.astype(np.float64)).astype(f32))
+        else:
+            raise ValueError(f"unknown activation {op}")
+        return round_to_dtype(r.astype(f32), dtype)
+
+    if gate is None:
+        return f(x)
+    return round_to_dtype((_f32(x) * f(gate)).astype(np.float32), dtype)
+
+
 def group_amax(w, group: int) -> np.ndarray:
     """|w| maxima over runs of ``group`` input channels: (N, K) -> (N, K / group).
     Group-wise weight scales are not in the reference (its weight scales are per

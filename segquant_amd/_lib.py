@@ -32,6 +32,7 @@ class QuantDesc(C.Structure):
         ("kseg_stride", C.c_int64),
         ("n_kseg", C.c_int32), ("dual", C.c_int32), ("dual_kseg_mask", C.c_uint32), ("dynamic", C.c_int32),
         ("kseg_bounds", C.c_int64 * (SEGQ_MAX_KSEG + 1)),
+        ("pre_op", C.c_int32), ("gate", C.c_void_p), ("ld_gate", C.c_int64),
     ]
 
 

@@ -21,6 +21,9 @@ struct QuantParams {
     int32_t n_kseg, dual, dynamic;
     uint32_t dual_mask;
     float scale_imm;  // used when scale == nullptr (one scale passed by value)
+    int32_t pre_op;   // segq_pre_op applied to the input before it is quantised
+    const void* gate; // with a pre_op: x is multiplied by op(gate) instead of being replaced by op(x)
+    int64_t ldg;
     int32_t kb[SEGQ_MAX_KSEG + 1];
 };
 
@@ -54,6 +57,39 @@ __device__ __forceinline__ void load16(const void* p, float (&v)[16]) {
             }
         }
     }
+}
+
+// ---- the producer's activation function, fused -----------------------------
+// What the layer in front of the linear would have written to memory in the
+// tensor's own dtype: op(x), or x * op(gate), each result rounded to that dtype
+// (torch evaluates these in fp32 and rounds once per operator).  The formulas
+// are torch's: gelu(tanh) = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))),
+// gelu = 0.5 x (1 + erf(x / sqrt 2)), silu = x / (1 + exp(-x)).
+// The transcendental parts run on the hardware's exp2 and reciprocal (an ulp
+// each) instead of the math library's tanhf / erff / expf, which cost ~50
+// instruction slots per element and made the fused kernel slower than the
+// separate activation kernel it replaces:
+//   0.5 (1 + tanh(u)) = 1 / (1 + e^(-2u))   (torch's 1 + tanhf(u) cancels for u < 0 and
+//   carries an absolute error of an ulp of 1 there; this form keeps the relative accuracy)
+//   1 + erf(z) = q or 2 - q for z < 0 or not, q = erfc(|z|) by Abramowitz and
+//   Stegun 7.1.26 (absolute error below 1.5e-7; no cancellation for z < 0)
+// Both are far inside a quantisation step of the codes they feed.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
+__device__ __forceinline__ float act_value(int op, float x) {
+    if (op == SEGQ_PRE_GELU_TANH) {
+        // 0.5 x (1 + tanh u) = x / (1 + e^(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3): nothing cancels
+        const float w = x * (1.0f + 0.044715f * (x * x));
+        return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w * -2.3022081986f));  // 2 sqrt(2/pi) log2(e)
+    }
+    if (op == SEGQ_PRE_GELU) {
+        const float z = fabsf(x) * 0.7071067811865476f;
+        const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+        const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+        const float q = poly * fast_exp(-z * z);
+        return x * 0.5f * (x < 0.0f ? q : 2.0f - q);
+    }
+    return x * __builtin_amdgcn_rcpf(1.0f + fast_exp(-x));  // SEGQ_PRE_SILU
 }
 
 // clamp first, then round half to even; a NaN operand is dropped by fmaxf and
@@ -145,26 +181,6 @@ __device__ __forceinline__ int kseg_of(const QuantParams& p, int col) {
     return s;
 }
 
-// ---- static scales ---------------------------------------------------------
-template <int DT, int FMT>
-__global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) {
-    const int64_t cpr = p.cols >> 4;  // runs of 16 per row
-    const int64_t run = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (run >= p.rows * cpr) return;
-    const int64_t row = run / cpr;
-    const int col = (int)(run - row * cpr) << 4;
-    const int ks = kseg_of(p, col);
-    const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
-    const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
-    const float s_pos = p.scale ? p.scale[si] : p.scale_imm;
-    const float s_neg = dual ? p.scale_neg[si] : s_pos;
-    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
-    float x[16];
-    load16<DT>(static_cast<const uint8_t*>(p.x) + (row * p.ldx + col) * esz, x);
-    // the second tensor exists only for DualScale column segments
-    encode16<FMT>(p, row, col, x, s_pos, s_neg, dual && p.codes_neg != nullptr);
-}
-
 // ---- dynamic per-row scales ------------------------------------------------
 template <int FMT>
 __device__ __forceinline__ float qmax_pos() {
@@ -213,6 +229,61 @@ __device__ __forceinline__ void raw_to_f32(const RawRun<DT>& r, float (&v)[16]) 
     }
 }
 
+// 16 fp32 values -> a run in the tensor's dtype, rounded to nearest even
+template <int DT>
+__device__ __forceinline__ void f32_to_raw(const float (&v)[16], RawRun<DT>& r) {
+    if constexpr (DT == SEGQ_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            r.q[i] = make_uint4(__float_as_uint(v[4 * i]), __float_as_uint(v[4 * i + 1]), __float_as_uint(v[4 * i + 2]),
+                                __float_as_uint(v[4 * i + 3]));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = (DT == SEGQ_BF16) ? pack2_bf16(v[8 * i + 2 * j], v[8 * i + 2 * j + 1])
+                                         : pack2_f16(v[8 * i + 2 * j], v[8 * i + 2 * j + 1]);
+            r.q[i] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
+// r holds 16 elements of x at (row, col); on return it holds what is quantised:
+// op(x), or x * op(gate), each operator's result rounded to the tensor's dtype
+template <int DT>
+__device__ __forceinline__ void pre_run(const QuantParams& p, int64_t row, int64_t col, RawRun<DT>& r) {
+    float v[16];
+    raw_to_f32<DT>(r, v);
+    if (p.gate) {
+        const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+        RawRun<DT> gr;
+        load_raw<DT>(static_cast<const uint8_t*>(p.gate) + (row * p.ldg + col) * esz, gr);
+        float g[16];
+        raw_to_f32<DT>(gr, g);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) g[i] = act_value(p.pre_op, g[i]);
+        f32_to_raw<DT>(g, gr);
+        raw_to_f32<DT>(gr, g);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] *= g[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = act_value(p.pre_op, v[i]);
+    }
+    f32_to_raw<DT>(v, r);
+}
+
+// With a fused activation the run kept in registers is the activation's output
+// (already in the tensor's dtype, so repacking it loses nothing).
+template <int DT, bool PRE>
+__device__ __forceinline__ void load_run(const QuantParams& p, const uint8_t* xrow, int64_t row, int c, RawRun<DT>& r) {
+    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+    load_raw<DT>(xrow + (size_t)c * 16 * esz, r);
+    if constexpr (PRE) pre_run<DT>(p, row, (int64_t)c << 4, r);
+}
+
 // Running maxima of the positive and of the negative side (strict masks x > 0 and
 // x < 0, segquant/quantizers/quantizer.py:172-189; NaN is ignored).  Without
 // DualScale only their maximum matters, which is one max of |x| per element.
@@ -239,7 +310,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // the row are issued before anything is computed; up to CACHE runs per thread
 // stay in registers in packed form between the reduction and the encode, longer
 // rows are read again (they hit in L2).
-template <int DT, int FMT, bool DUAL>
+template <int DT, int FMT, bool DUAL, bool PRE>
 __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p) {
     constexpr int CACHE = 4;
     __shared__ float red[2][4];
@@ -255,7 +326,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
 #pragma unroll
         for (int i = 0; i < CACHE; ++i) {
             const int c = c0 + threadIdx.x + i * 256;
-            if (c < c1) load_raw<DT>(xrow + (size_t)c * 16 * esz, raw[i]);
+            if (c < c1) load_run<DT, PRE>(p, xrow, row, c, raw[i]);
         }
         float amax_p = 0.0f, amax_n = 0.0f;
 #pragma unroll
@@ -270,7 +341,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
         for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
             RawRun<DT> t;
             float v[16];
-            load_raw<DT>(xrow + (size_t)c * 16 * esz, t);
+            load_run<DT, PRE>(p, xrow, row, c, t);
             raw_to_f32<DT>(t, v);
             track_amax<DUAL>(v, amax_p, amax_n);
         }
@@ -308,7 +379,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
         for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
             RawRun<DT> t;
             float v[16];
-            load_raw<DT>(xrow + (size_t)c * 16 * esz, t);
+            load_run<DT, PRE>(p, xrow, row, c, t);
             raw_to_f32<DT>(t, v);
             encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
         }
@@ -319,7 +390,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
 // For rows of up to 64 * CPL runs: the whole row is in flight at once, the
 // maximum is reduced with cross-lane shuffles only, and four rows share a
 // workgroup without ever synchronising.
-template <int DT, int FMT, int CPL, bool DUAL>
+template <int DT, int FMT, int CPL, bool DUAL, bool PRE>
 __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantParams p) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -335,7 +406,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
 #pragma unroll
         for (int i = 0; i < CPL; ++i) {
             const int c = c0 + lane + i * 64;
-            if (c < c1) load_raw<DT>(xrow + (size_t)c * 16 * esz, raw[i]);
+            if (c < c1) load_run<DT, PRE>(p, xrow, row, c, raw[i]);
         }
         float amax_p = 0.0f, amax_n = 0.0f;
 #pragma unroll
@@ -373,6 +444,33 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
     }
 }
 
+// ---- static scales ---------------------------------------------------------
+template <int DT, int FMT, bool PRE>
+__global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) {
+    const int64_t cpr = p.cols >> 4;  // runs of 16 per row
+    const int64_t run = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (run >= p.rows * cpr) return;
+    const int64_t row = run / cpr;
+    const int col = (int)(run - row * cpr) << 4;
+    const int ks = kseg_of(p, col);
+    const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
+    const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
+    const float s_pos = p.scale ? p.scale[si] : p.scale_imm;
+    const float s_neg = dual ? p.scale_neg[si] : s_pos;
+    const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+    float x[16];
+    if constexpr (PRE) {
+        RawRun<DT> r;
+        load_raw<DT>(static_cast<const uint8_t*>(p.x) + (row * p.ldx + col) * esz, r);
+        pre_run<DT>(p, row, col, r);
+        raw_to_f32<DT>(r, x);
+    } else {
+        load16<DT>(static_cast<const uint8_t*>(p.x) + (row * p.ldx + col) * esz, x);
+    }
+    // the second tensor exists only for DualScale column segments
+    encode16<FMT>(p, row, col, x, s_pos, s_neg, dual && p.codes_neg != nullptr);
+}
+
 // ---- fake e4m3 round trip ----------------------------------------------------
 __device__ __forceinline__ float e4m3_roundtrip(float v) {
     int r = __builtin_amdgcn_cvt_pk_fp8_f32(sat_e4m3(v), 0.0f, 0, false);
@@ -395,22 +493,27 @@ __global__ void __launch_bounds__(256) fake_e4m3_kernel(const void* x, void* out
 }
 
 // ---- host side ---------------------------------------------------------------
-template <int DT, int FMT>
+template <int DT, int FMT, bool PRE>
 static int launch_quant(const QuantParams& p, hipStream_t st) {
     if (p.dynamic) {
         int longest = 0;  // runs of 16 in the longest column segment
         for (int i = 0; i < p.n_kseg; ++i) longest = longest > (p.kb[i + 1] - p.kb[i]) / 16 ? longest : (p.kb[i + 1] - p.kb[i]) / 16;
         const dim3 wgrid((unsigned)((p.rows + 3) / 4)), bgrid((unsigned)p.rows);
         if (longest <= 64 * 4) {
-            if (p.dual) hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, true>), wgrid, dim3(256), 0, st, p);
-            else hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, false>), wgrid, dim3(256), 0, st, p);
+            if (p.dual) hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, true, PRE>), wgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 4, false, PRE>), wgrid, dim3(256), 0, st, p);
+        } else if (longest <= 64 * 8 && longest % 256 != 0) {
+            // rows a workgroup's 256 threads would share unevenly (320 runs: a quarter of the threads
+            // with two, the rest with one) stay with one wave per row
+            if (p.dual) hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 8, true, PRE>), wgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((quant_dynamic_wave_kernel<DT, FMT, 8, false, PRE>), wgrid, dim3(256), 0, st, p);
         } else {
-            if (p.dual) hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, true>), bgrid, dim3(256), 0, st, p);
-            else hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, false>), bgrid, dim3(256), 0, st, p);
+            if (p.dual) hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, true, PRE>), bgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((quant_dynamic_kernel<DT, FMT, false, PRE>), bgrid, dim3(256), 0, st, p);
         }
     } else {
         const int64_t runs = p.rows * (p.cols >> 4);
-        hipLaunchKernelGGL((quant_static_kernel<DT, FMT>), dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((quant_static_kernel<DT, FMT, PRE>), dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, st, p);
     }
     return check_launch("segq_quantize");
 }
@@ -418,9 +521,9 @@ static int launch_quant(const QuantParams& p, hipStream_t st) {
 template <int DT>
 static int launch_quant_fmt(const QuantParams& p, hipStream_t st) {
     switch (p.fmt) {
-        case SEGQ_CODE_I8: return launch_quant<DT, SEGQ_CODE_I8>(p, st);
-        case SEGQ_CODE_E4M3: return launch_quant<DT, SEGQ_CODE_E4M3>(p, st);
-        case SEGQ_CODE_I4: return launch_quant<DT, SEGQ_CODE_I4>(p, st);
+        case SEGQ_CODE_I8: return p.pre_op ? launch_quant<DT, SEGQ_CODE_I8, true>(p, st) : launch_quant<DT, SEGQ_CODE_I8, false>(p, st);
+        case SEGQ_CODE_E4M3: return p.pre_op ? launch_quant<DT, SEGQ_CODE_E4M3, true>(p, st) : launch_quant<DT, SEGQ_CODE_E4M3, false>(p, st);
+        case SEGQ_CODE_I4: return p.pre_op ? launch_quant<DT, SEGQ_CODE_I4, true>(p, st) : launch_quant<DT, SEGQ_CODE_I4, false>(p, st);
     }
     return fail(SEGQ_ERR_ARG, "segq_quantize: unknown code_fmt %d", p.fmt);
 }
@@ -461,6 +564,13 @@ int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_b
     p.n_kseg = d->n_kseg; p.dual = d->dual ? 1 : 0; p.dynamic = d->dynamic ? 1 : 0;
     p.dual_mask = d->dual_kseg_mask;
     p.scale_imm = scale_by_value ? *scale_by_value : 0.0f;
+    if (d->pre_op < SEGQ_PRE_NONE || d->pre_op > SEGQ_PRE_SILU) return fail(SEGQ_ERR_ARG, "segq_quantize: unknown pre_op %d", d->pre_op);
+    if (d->gate) {
+        if (d->pre_op == SEGQ_PRE_NONE) return fail(SEGQ_ERR_ARG, "segq_quantize: a gate needs a pre_op");
+        if (d->ld_gate < d->cols || (d->ld_gate * esz) % 16 || !aligned16(d->gate))
+            return fail(SEGQ_ERR_ARG, "segq_quantize: gate must be 16-byte aligned with ld_gate >= cols");
+    }
+    p.pre_op = d->pre_op; p.gate = d->gate; p.ldg = d->ld_gate;
     if (d->n_kseg == 1) {
         p.kb[0] = 0; p.kb[1] = (int32_t)d->cols;
     } else {

@@ -166,10 +166,24 @@ class SegmentLinear(nn.Module):
         if self.bias_data is not None:
             self.bias_data = self.bias_data.to(self.origin_device)
 
-    def forward(self, x, chunked=False):
+    @staticmethod
+    def _activated(x, pre_op, gate):
+        """op(x), or x * op(gate), with torch operators (the routes without the fused kernel)."""
+        import torch.nn.functional as F
+        fn = {"gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "gelu": F.gelu, "silu": F.silu}[pre_op]
+        return fn(x) if gate is None else x * fn(gate)
+
+    def forward(self, x, chunked=False, pre_op=None, gate=None):
+        """``pre_op`` ("gelu_tanh", "gelu", "silu") and ``gate`` are not in the reference: they
+        hand the activation function of the module in front (x -> op(x), or x * op(gate) for
+        GEGLU / SwiGLU, backend/torch/layers/activations.py:52-57, :77-80, :110-121) to this
+        layer, whose quantise kernel evaluates it on the fly instead of reading back a stored
+        activation tensor.  The layer must have been calibrated on the activated input."""
         opt = self.optimizer
         if not chunked and opt.real_quant and opt.has_calibrated:
-            return opt.forward_fused(x, self.bias_data if self.bias else None)
+            return opt.forward_fused(x, self.bias_data if self.bias else None, pre_op=pre_op, gate=gate)
+        if pre_op is not None:
+            x = self._activated(x, pre_op, gate)
         if not chunked and not self.equal_chunks:
             res = opt.forward_fake(x)
             return res + self.bias_data if self.bias else res

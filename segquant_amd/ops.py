@@ -86,6 +86,10 @@ def _launch(kind, info, fn):
     return rc
 
 
+# enum segq_pre_op
+PRE_OPS = {"gelu_tanh": 1, "gelu": 2, "silu": 3}
+
+
 def code_dtype(fmt: str) -> torch.dtype:
     """Storage dtype of codes: int8 as int8, e4m3 and packed int4 as uint8
     (segquant/src/real_quant/seg_utils.h:25-45)."""
@@ -100,15 +104,18 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
              kseg_bounds: Optional[Sequence[int]] = None, kseg_stride: int = 0,
              dual: bool = False, dual_kseg_mask: int = 0xFFFFFFFF, dynamic: bool = False,
              two_tensors: bool = False, out: Optional[torch.Tensor] = None,
-             out_neg: Optional[torch.Tensor] = None):
+             out_neg: Optional[torch.Tensor] = None, pre_op: Optional[str] = None,
+             gate: Optional[torch.Tensor] = None):
     """Quantise a 2-D float matrix ``x`` (rows, cols) to codes.
 
     See ``segq_quantize`` in include/segq.h for the scale indexing.  Returns the
     code tensor, or ``(Xp, Xn)`` when ``two_tensors`` (DualScale in the
     reference's two-tensor layout).  With ``dynamic`` the scale tensors are
-    written by the kernel.
+    written by the kernel.  ``pre_op`` ("gelu_tanh", "gelu", "silu") fuses the
+    activation function in front of the linear: op(x) is quantised, or
+    x * op(gate) when ``gate`` (same shape and dtype as ``x``) is given.
     """
-    _need_cuda(x, scale, scale_neg)
+    _need_cuda(x, scale, scale_neg, gate)
     if x.dim() != 2 or x.stride(1) != 1:
         raise RuntimeError("quantize expects a 2-D tensor with a contiguous last dimension")
     rows, cols = x.shape
@@ -135,8 +142,16 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
         for i, b in enumerate(kseg_bounds):
             d.kseg_bounds[i] = int(b)
     d.dual = 1 if dual else 0; d.dual_kseg_mask = dual_kseg_mask & 0xFFFFFFFF; d.dynamic = 1 if dynamic else 0
-    info = dict(rows=rows, cols=cols, x_bytes=x.element_size(), code_bytes=0.5 if fmt == FMT_INT4 else 1.0,
-                tensors=2 if two_tensors else 1, dynamic=bool(dynamic))
+    if pre_op is not None:
+        if pre_op not in PRE_OPS:
+            raise RuntimeError(f"pre_op must be one of {sorted(PRE_OPS)}")
+        d.pre_op = PRE_OPS[pre_op]
+    if gate is not None:
+        if pre_op is None or gate.shape != x.shape or gate.dtype != x.dtype or gate.stride(1) != 1:
+            raise RuntimeError("gate needs a pre_op and the shape, dtype and contiguous rows of x")
+        d.gate = gate.data_ptr(); d.ld_gate = gate.stride(0) if rows > 1 else cols
+    info = dict(rows=rows, cols=cols, x_bytes=x.element_size() * (2 if gate is not None else 1),
+                code_bytes=0.5 if fmt == FMT_INT4 else 1.0, tensors=2 if two_tensors else 1, dynamic=bool(dynamic))
     L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
     return (out, out_neg) if two_tensors else out
 

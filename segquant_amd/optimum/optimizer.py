@@ -253,16 +253,24 @@ class DefaultOptimizer(BaseOptimizer):
                           sw_cs=1 if sw_vec.numel() > 1 else 0, bounds=bounds, N=N, K=K)
         return self._plan
 
-    def forward_fused(self, x: torch.Tensor, bias=None) -> torch.Tensor:
+    def forward_fused(self, x: torch.Tensor, bias=None, pre_op=None, gate=None) -> torch.Tensor:
         """Final (..., out) result in ``x.dtype``: quantise + segmented GEMM with
         de-quantisation and bias fused.  Equivalent to ``forward`` followed by
         the recombination of ``SegmentLinear.forward``, with the partial sums of
-        input segments combined in fp32 and rounded once."""
+        input segments combined in fp32 and rounded once.
+
+        ``pre_op`` / ``gate``: the layer's input is op(x), or x * op(gate), with
+        the activation function evaluated inside the quantise kernel (see
+        ``ops.quantize``); the scales must have been calibrated on that input."""
         plan = self._plan or self._build_plan(x.device)
         K, N = plan["K"], plan["N"]
         x2 = x.reshape(-1, K)
         if not x2.is_contiguous():
             x2 = x2.contiguous()
+        if gate is not None:
+            gate = gate.reshape(-1, K)
+            if not gate.is_contiguous():
+                gate = gate.contiguous()
         M = x2.shape[0]
         S = self.chunks if self.seg_mode == "input" else 1
         bounds = plan["bounds"]
@@ -294,7 +302,7 @@ class DefaultOptimizer(BaseOptimizer):
         # registers), measured on the 4608 x 15360 x 3072 shape.
         codes = ops.quantize(x2, plan["fa"], pos, neg, row_stride=1 if per_tok else 0,
                              kseg_bounds=bounds if S > 1 else None, kseg_stride=kstride, dual=dual,
-                             dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual)
+                             dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual, pre_op=pre_op, gate=gate)
         codes, codes_neg = codes if dual else (codes, None)
         ranges = []
         for s in range(S):

@@ -352,6 +352,54 @@ def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
     assert (y0 - y1).abs().max().item() <= 2e-6 * y0.abs().max().item()
 
 
+@pytest.mark.parametrize("op", ["gelu_tanh", "gelu", "silu"])
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("dt", ["bf16", "fp32", "fp16"])
+def test_quantize_with_fused_activation(ops, op, gated, dt):
+    """op(x), or x * op(gate), evaluated inside the quantise kernel.  The kernel's tanhf /
+    erff / expf may be an ulp off the oracle's correctly rounded ones, which moves a value
+    across a rounding boundary now and then: codes may differ by one step on a small
+    fraction of the elements, never by more.  Static per-tensor scale with DualScale into two
+    tensors (wave-per-row and workgroup-per-row shapes do not matter here), then dynamic
+    per-row scales on both dynamic kernels, checked with the scales the kernel reports."""
+    import torch.nn.functional as F
+    tdt = TDT[dt]
+    for rows, cols in ((33, 1024), (9, 4608)):
+        g = torch.Generator().manual_seed(41)
+        x = (torch.randn(rows, cols, generator=g) * 2.5).to(tdt)
+        gate = (torch.randn(rows, cols, generator=g) * 2).to(tdt) if gated else None
+        xd, gd = x.to(DEV), (gate.to(DEV) if gated else None)
+        want_act = O.activation(x.float().numpy(), op, gate=gate.float().numpy() if gated else None, dtype=dt)
+        # the same thing from torch's own operators on the device: a second, independent check
+        fn = {"gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "gelu": F.gelu, "silu": F.silu}[op]
+        torch_act = fn(xd) if not gated else xd * fn(gd)
+        pa, na = O.dual_amax(want_act)
+        ps, ns = O.int_dual_scales(pa, na, 8)
+        sp, sn = torch.tensor([ps], device=DEV), torch.tensor([ns], device=DEV)
+        cp, cn = ops.quantize(xd, O.FMT_INT8, sp, sn, dual=True, two_tensors=True, pre_op=op, gate=gd)
+        wp, wn = O.quantize_act_dual(want_act[None], np.float32([ps]), np.float32([ns]), O.FMT_INT8)
+        tp, tn = ops.quantize(torch_act, O.FMT_INT8, sp, sn, dual=True, two_tensors=True)
+        for got, want, tor in ((cp, wp[0], tp), (cn, wn[0], tn)):
+            d = np.abs(got.cpu().numpy().astype(np.int32) - want.astype(np.int32))
+            assert d.max() <= 1 and (d != 0).mean() <= 4e-3, (d.max(), (d != 0).mean())
+            dt_ = (got.int() - tor.int()).abs()
+            assert dt_.max().item() <= 1 and (dt_ != 0).float().mean().item() <= 4e-3
+        # dynamic per-row scales, e4m3 codes
+        scale = torch.empty(rows, device=DEV)
+        c = ops.quantize(xd, O.FMT_E4M3, scale, row_stride=1, dynamic=True, pre_op=op, gate=gd)
+        want_scale = O.row_scale_div(np.abs(want_act).max(axis=1), 448.0)
+        got_scale = scale.cpu().numpy()
+        assert (np.abs(got_scale - want_scale) <= 2.0 ** -6 * want_scale).all()  # an ulp of the row's largest value
+        wc = O.quantize_act(want_act[None], got_scale, O.FMT_E4M3)[0]
+        # (e4m3 keeps three mantissa bits however small the value, so the negative tail of the
+        # gelus, where fp32 evaluations of 1 + tanh / 1 + erf carry cancellation noise, lands on
+        # neighbouring codes far more often than with the integer codes above)
+        same = c.cpu().numpy() == wc
+        assert same.mean() >= 1 - 2e-2
+        v_got, v_want = O.e4m3_decode(c.cpu().numpy()), O.e4m3_decode(wc)
+        assert (np.abs(v_got - v_want) <= 0.126 * np.abs(v_want) + 2.0 ** -9).all()  # neighbouring e4m3 values
+
+
 @pytest.mark.parametrize("fmt_w", [O.FMT_INT4, O.FMT_INT8])
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
 def test_group_wise_weight_scales(ops, fmt_w, dt):

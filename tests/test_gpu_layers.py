@@ -238,6 +238,28 @@ def test_quantize_real_vs_fake_like_the_reference_grid(atype, wtype, axis, model
     assert ((a - c).norm() / a.norm()).item() < (0.25 if wtype == "INT4" else 0.08)
 
 
+@pytest.mark.parametrize("op,gated", [("gelu_tanh", False), ("gelu", True), ("silu", True)])
+def test_layer_with_the_activation_function_fused_into_its_quantise_kernel(op, gated):
+    """forward(x, pre_op=...) == forward(op(x)) with torch's operator, to the rounding of the
+    output dtype (a code may move by one step where the two tanh / erf / exp differ by an ulp),
+    on the DualScale e4m3 MLP of config 2 and on the fake path of the same layer."""
+    from segquant_amd import workloads as W
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    spec = [s for s in W.config_linears(2, M=192) if s.name == "fc2"][0]
+    g = torch.Generator().manual_seed(7)
+    pre = (torch.randn(192, spec.K, generator=g) * 1.5).to(torch.bfloat16).to(DEV)
+    gate = (torch.randn(192, spec.K, generator=g) * 1.5).to(torch.bfloat16).to(DEV) if gated else None
+    act = SegmentLinear._activated(pre, op, gate)
+    layer, _ = W.build_layer(spec, device=DEV, real_quant=True, x=act.float().cpu())
+    want = layer(act).float()
+    got = layer(pre, pre_op=op, gate=gate).float()
+    assert (got - want).abs().max().item() <= 2e-2 * want.abs().max().item()
+    assert ((got - want).abs() > 2.0 ** -7 * want.abs().max()).float().mean().item() <= 1e-2
+    fake, _ = W.build_layer(spec, device=DEV, real_quant=False, x=act.float().cpu())
+    pre32, gate32 = pre.float(), (gate.float() if gated else None)  # the fake path multiplies in the weight's fp32
+    assert torch.equal(fake(pre32, pre_op=op, gate=gate32), fake(SegmentLinear._activated(pre32, op, gate32)))
+
+
 def test_unsupported_kernel_type_warns_and_uses_fake_path(capsys):
     from segquant_amd.layers.SegmentLinear import SegmentLinear
     lin = torch.nn.Linear(64, 32)

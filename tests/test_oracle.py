@@ -341,3 +341,31 @@ def test_linear_groups_against_bruteforce_and_per_row():
     np.testing.assert_allclose(O.linear_groups(a, b, sx, sw_same, g),
                                acc / (sx.astype(np.float64)[:, None] * sw_same[:, 0].astype(np.float64)[None, :]),
                                rtol=1e-12)
+
+
+# ---- activation functions fused into the quantise kernel ----------------------
+@pytest.mark.parametrize("op", ["gelu_tanh", "gelu", "silu"])
+@pytest.mark.parametrize("dt", ["fp32", "bf16", "fp16"])
+def test_activation_matches_torch_cpu_operators(op, dt):
+    """Library routine as the pin: torch's own operators on the CPU.  torch evaluates
+    in fp32 with its vectorised tanh / erf / exp, the oracle in fp64: they may differ
+    by an ulp of the tensor's dtype at rounding boundaries, nowhere by more."""
+    import torch.nn.functional as F
+    tdt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dt]
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(64, 256, generator=g) * 3).to(tdt)
+    x[0, :6] = torch.tensor([0.0, -0.0, 20.0, -20.0, 1e-3, -1e-3]).to(tdt)
+    gate = (torch.randn(64, 256, generator=g) * 2).to(tdt)
+    fn = {"gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "gelu": F.gelu, "silu": F.silu}[op]
+    ulp = {"fp32": 2.0 ** -21, "bf16": 2.0 ** -6, "fp16": 2.0 ** -9}[dt]  # two ulps at the bottom of a binade
+    xf, gf = x.float().numpy(), gate.float().numpy()
+    # where 1 + tanh(.) or 1 + erf(.) cancels, an error of a few ulps in the function (torch's
+    # vectorised erf is that far off) is an absolute error of ~1e-6 |argument|
+    for want, got, slack in ((fn(x), O.activation(xf, op, dtype=dt), 1e-6 * np.abs(xf)),
+                             (x * fn(gate), O.activation(xf, op, gate=gf, dtype=dt), 1e-6 * np.abs(gf) * np.abs(xf))):
+        want = want.float().numpy()
+        diff = np.abs(got - want)
+        assert (diff <= ulp * np.abs(want) + slack + 1e-30).all()
+    # closed-form anchors: gelu(0) = silu(0) = 0, large |x| -> x or 0, odd/even structure
+    z = O.activation(np.array([0.0, 30.0, -30.0], dtype=np.float32), op)
+    assert z[0] == 0.0 and z[1] == 30.0 and abs(z[2]) < 1e-6
