@@ -61,13 +61,15 @@ class RealQuantExt:
     @staticmethod
     def _scaled(fa, fw):
         def fn(inputs, weights, scale_x, scale_w):
-            return ops.real_quantized_gemm_scaled(fa, fw, inputs, weights, scale_x, scale_w)
+            from .. import torch_ops
+            return torch_ops.real_quantized_gemm_scaled(inputs, weights, scale_x, scale_w, fa, fw)
         return fn
 
     @staticmethod
     def _dual(fa, fw):
         def fn(inputs, weights, pos_scale_x, neg_scale_x, scale_w):
-            return ops.real_quantized_gemm_dual_scaled(fa, fw, inputs, weights, pos_scale_x, neg_scale_x, scale_w)
+            from .. import torch_ops
+            return torch_ops.real_quantized_gemm_dual_scaled(inputs, weights, pos_scale_x, neg_scale_x, scale_w, fa, fw)
         return fn
 
     def create_quantized_weights(self, x: torch.Tensor) -> torch.Tensor:

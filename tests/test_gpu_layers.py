@@ -260,6 +260,31 @@ def test_layer_with_the_activation_function_fused_into_its_quantise_kernel(op, g
     assert torch.equal(fake(pre32, pre_op=op, gate=gate32), fake(SegmentLinear._activated(pre32, op, gate32)))
 
 
+def test_reference_named_operators_trace_and_compile():
+    """The chunked route calls the reference-named operator through torch.library: opcheck's
+    schema / fake-tensor / dispatch checks pass, and a compiled function that calls it gives
+    the eager result without a graph break."""
+    from segquant_amd import torch_ops  # noqa: F401
+    g = torch.Generator().manual_seed(3)
+    S, M, N, K = 2, 48, 64, 128
+    x = torch.randn(S, M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randint(-127, 128, (S, N, K), generator=g, dtype=torch.int8).to(DEV)
+    sx = (torch.rand(S * M, generator=g) * 20 + 5).to(DEV)
+    sw = (torch.rand(S, generator=g) * 50 + 5).to(DEV)
+    op = torch.ops.segquant_amd.real_quantized_gemm_scaled
+    torch.library.opcheck(op, (x, w, sx, sw, "int8", "int8"),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    torch.library.opcheck(torch.ops.segquant_amd.real_quantized_gemm_dual_scaled, (x, w, sx, sx * 2, sw, "int8", "int8"),
+                          test_utils=("test_schema", "test_faketensor"))
+
+    def f(x, w, sx, sw):
+        return op(x, w, sx, sw, "int8", "int8").float().sum(0) * 0.5
+
+    want = f(x, w, sx, sw)
+    got = torch.compile(f, backend="aot_eager", fullgraph=True)(x, w, sx, sw)
+    assert torch.equal(got, want)
+
+
 def test_unsupported_kernel_type_warns_and_uses_fake_path(capsys):
     from segquant_amd.layers.SegmentLinear import SegmentLinear
     lin = torch.nn.Linear(64, 32)

@@ -352,3 +352,35 @@ def test_torch_fake_path_equals_numpy_oracle():
             wf = O.fake_quant_int(w.numpy(), np.float32(sw))
         want = xf @ wf.T
         assert np.abs(y - want).max() <= 2e-6 * np.abs(want).max()
+
+
+# ------------------------------------------------------------------ traceable operators
+def test_custom_operators_have_shape_only_kernels_for_tracing():
+    """The reference-named operators are torch.library custom ops: on meta / fake tensors they
+    return the contract's output shape and dtype without touching a GPU, and a symbolic trace
+    keeps them as single nodes."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from segquant_amd import torch_ops  # noqa: F401  (registers the operators)
+    x = torch.empty(3, 2, 5, 64, device="meta", dtype=torch.bfloat16)
+    w8 = torch.empty(3, 48, 64, device="meta", dtype=torch.int8)
+    w4 = torch.empty(3, 48 * 64 // 2, device="meta", dtype=torch.uint8)
+    s = torch.empty(3, device="meta")
+    o = torch.ops.segquant_amd.real_quantized_gemm_scaled(x, w8, s, s, "int8", "int8")
+    assert o.shape == (3, 2, 5, 48) and o.dtype == torch.bfloat16 and o.device.type == "meta"
+    o = torch.ops.segquant_amd.real_quantized_gemm_dual_scaled(x, w4, s, s, s, "int8", "int4")
+    assert o.shape == (3, 2, 5, 48) and o.dtype == torch.bfloat16
+
+    def f(x, w, sx, sw):
+        return torch.ops.segquant_amd.real_quantized_gemm_scaled(x * 2, w, sx, sw, "fpe4m3", "fpe4m3").sum(0)
+
+    with FakeTensorMode() as mode:
+        args = [mode.from_tensor(t) for t in (torch.zeros(3, 5, 64), torch.zeros(3, 48, 64, dtype=torch.uint8),
+                                              torch.ones(3), torch.ones(3))]
+        g = make_fx(f)(*args)
+    targets = [n.target for n in g.graph.nodes if n.op == "call_function"]
+    assert torch.ops.segquant_amd.real_quantized_gemm_scaled.default in targets
+    # real CPU tensors have no kernel: the call fails loudly
+    with pytest.raises(RuntimeError):
+        torch.ops.segquant_amd.real_quantized_gemm_scaled(torch.zeros(1, 2, 16), torch.zeros(1, 4, 16, dtype=torch.int8),
+                                                          torch.ones(1), torch.ones(1), "int8", "int8")
