@@ -205,6 +205,10 @@ typedef struct segq_gemm_desc {
                          * a small kernel and the int8 GEMM kernels run on that (same accumulators, bit for bit;
                          * worth it when m is large and the GEMM is bound by the matrix cores, not by reading b).
                          * NULL or too small: int4 weights are unpacked on their way into LDS inside the GEMM.
+                         * With int8 codes on both sides, several ranges, batch == 1 and tiles * tile_rows *
+                         * tile_cols * 4 bytes here (4 (m + 288) (n + 288) always suffices), the sums of finished
+                         * ranges are parked in the workspace as fp32 instead of in a second register set, which
+                         * keeps the largest tiles available (same result up to fp32 rounding order).
                          * Contents are undefined afterwards.  Replaces nothing in the reference, whose CUTLASS
                          * kernel converts int4 in registers (segquant/src/real_quant/real_gemm.cu:208-305). */
     int64_t workspace_bytes;

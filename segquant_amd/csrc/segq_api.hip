@@ -198,13 +198,31 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         p.grw = d->group_dequant;
         p.grw_gs = d->group_dequant_stride;
     }
+    // int8 with several ranges keeps the big tiles if the caller lends a workspace to park
+    // finished ranges in: one fp32 tile per workgroup
+    bool park = i8 && plain8 && fold && !groups && wide_ok && d->batch == 1 && d->out_dtype != SEGQ_ACC && d->workspace &&
+                al(d->workspace, 16);
+    auto park_fits = [&](int c) {
+        if (c < FIRST_WIDE_CFG || c > FIRST_WIDE_CFG + 5) return false;
+        const TileCfg& t = TILE_CFGS[c];
+        const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
+        return d->workspace_bytes >= tiles * t.bm * t.bn * 4;
+    };
     if (d->tile == 0) {
         if (groups) cfg = FIRST_WIDE_CFG + 3;  // the one tile the group kernel is built for
-        else cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
+        else {
+            cfg = park ? choose_tile(d->m, d->n, d->batch, false, wide_ok, plain8) : -1;
+            park = park && park_fits(cfg);
+            if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
+        }
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
-    if (cfg >= FIRST_WIDE_CFG) {
+    if (d->tile != 0) park = park && park_fits(cfg);
+    if (park) p.park = static_cast<float*>(d->workspace);
+    if (park) {
+        // every 8-wave tile serves several ranges this way
+    } else if (cfg >= FIRST_WIDE_CFG) {
         if (!wide_ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs K ranges in multiples of 128", cfg + 1);
         if (fold2 && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
         if (groups && cfg != FIRST_WIDE_CFG + 3)

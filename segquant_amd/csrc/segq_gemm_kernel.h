@@ -46,6 +46,7 @@ struct GemmParams {
     int32_t tiles_m, tiles_n, group_m;
     int32_t vec_store;    // output rows allow 4-element vector stores
     int32_t vec_store16;  // 16-bit output rows allow 16-byte stores
+    float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
     const float* grw;     // group-wise de-quantisation factors [K / 128][grw_gs], or null
     int64_t grw_gs;
     KRange r[SEGQ_MAX_RANGES];

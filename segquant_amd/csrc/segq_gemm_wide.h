@@ -431,7 +431,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
 // s_waitcnt immediate for "vmcnt(n) lgkmcnt(0)" on gfx9-family encodings
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }
 
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmParams p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -458,7 +458,17 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // (two int32 sets taking turns, so that the conversion spreads over the whole
     // step, measured no faster: the kernel is held by its one workgroup per CU).
     static_assert(!GRP || (!F8 && NS == 2), "group factors: int8, two stages");
-    constexpr bool ACCF = FOLD && !F8 && !GRP;
+    //
+    // PARK (int8, several ranges): no second register set at all.  When a range
+    // ends, its int32 sums are converted to the LAST range's units
+    // (x sx_L sw_L / (sx sw)) and added to this tile's fp32 slot of a workspace
+    // the caller lends; the accumulators restart from zero.  The epilogue adds the
+    // slot to the last range's sums and scales once.  Each thread only ever reads
+    // back what it wrote itself.  This keeps the big tiles for int8 with K
+    // segments or DualScale: a few hundred KB of traffic per tile and range
+    // boundary against ~14 MB of operands.
+    static_assert(!PARK || (FOLD && !F8 && !GRP), "parking: int8 with several ranges");
+    constexpr bool ACCF = FOLD && !F8 && !GRP && !PARK;
     constexpr bool HASF = ACCF || GRP;
     const acc_t acc_zero = {0, 0, 0, 0};
 
@@ -594,6 +604,46 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 for (int b = 0; b < TM; ++b) {
                     accf[a][b] += __builtin_convertvector(set[a][b], v4f) * g;
                     set[a][b] = acc_zero;
+                }
+            }
+        }
+    };
+    v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + (int64_t)blockIdx.x * (BM * BN / 4) + tid : nullptr;
+    auto park = [&](int r) __attribute__((always_inline)) {
+        if constexpr (PARK) {
+            if (r + 1 < p.nr) {
+                const int rl = p.nr - 1;
+                const float* sx = p.r[r].sx;
+                const float* sw = p.r[r].sw;
+                const float* sx2 = p.r[rl].sx;
+                const float* sw2 = p.r[rl].sw;
+                const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs, rs2 = p.r[rl].sx_rs, cs2 = p.r[rl].sw_cs;
+                float fx[TM];
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    const int64_t m = min(m_base + b * 16, p.M - 1);
+                    fx[b] = sx2[m * rs2] * __builtin_amdgcn_rcpf(sx[m * rs]);
+                }
+#pragma unroll
+                for (int a = 0; a < TN; ++a) {
+                    v4f fw;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int64_t n = min(n_base + a * 16 + v, p.N - 1);
+                        fw[v] = sw2[n * cs2] * __builtin_amdgcn_rcpf(sw[n * cs]);
+                    }
+                    v4f old[TM];
+                    if (r > 0) {
+#pragma unroll
+                        for (int b = 0; b < TM; ++b) old[b] = slot[(a * TM + b) * NT];
+                    }
+#pragma unroll
+                    for (int b = 0; b < TM; ++b) {
+                        v4f t = __builtin_convertvector(acc[a][b], v4f) * (fw * fx[b]);
+                        if (r > 0) t += old[b];
+                        slot[(a * TM + b) * NT] = t;
+                        acc[a][b] = acc_zero;
+                    }
                 }
             }
         }
@@ -867,7 +917,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         cslot = (cslot + 1) & 3;
         if (ck >= ck1) {  // the range is complete: fold it, move to the next one
             if constexpr (GRP && FOLD) add_groups(acc, grw, pslot);  // this step's sums are still in the old range's units
-            if constexpr (FOLD) fold(cr);
+            if constexpr (PARK) park(cr);
+            else if constexpr (FOLD) fold(cr);
             ++cr;
             const int rr = min(cr, p.nr - 1);
             ck = p.r[rr].k0;
@@ -887,6 +938,24 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         add_groups(acc, grw, pslot);  // the last step's sums
         v4f none[1][1];
         wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, false>(p, accf, none, smem, z, m0, n0, wave, lane, r_epi, epi);
+    } else if constexpr (PARK) {
+        // the earlier ranges' sums come back in two halves, each with all its loads in flight at once
+        v4f accp[TN][TM];
+        constexpr int H = (TN + 1) / 2;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            v4f old[H][TM];
+#pragma unroll
+            for (int a = h * H; a < min(TN, (h + 1) * H); ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b) old[a - h * H][b] = slot[(a * TM + b) * NT];
+#pragma unroll
+            for (int a = h * H; a < min(TN, (h + 1) * H); ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b) accp[a][b] = __builtin_convertvector(acc[a][b], v4f) + old[a - h * H][b];
+        }
+        v4f none[1][1];
+        wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, false>(p, accp, none, smem, z, m0, n0, wave, lane, r_epi, epi);
     } else {
         wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, r_epi, epi);
     }
@@ -908,9 +977,9 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 }
 
 // wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false>
 int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
-    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP>;
+    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK>;
     // the stages, the epilogue's vectors, and the ring of group factors
     constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4 + (GRP ? 4 * BN * 4 : 0);
     static bool attr_set = false;
@@ -957,6 +1026,17 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 3: return launch_pipe_instance<128, 128, 4, 2, FMT, true, 2>(p, batch, st);
                     case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, true, 2>(p, batch, st);
                     case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, true, 2>(p, batch, st);
+                }
+            } else if (p.park) {  // int8, several ranges, a workspace to park finished ranges in: every tile
+                if constexpr (!F8W) {
+                    switch (wcfg) {
+                        case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, true, 2, false, true>(p, batch, st);
+                        case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2, false, true>(p, batch, st);
+                        case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2, false, true>(p, batch, st);
+                        case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, true, 2, false, true>(p, batch, st);
+                        case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, true, 2, false, true>(p, batch, st);
+                        case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, true, 2, false, true>(p, batch, st);
+                    }
                 }
             } else {
                 switch (wcfg) {

@@ -175,15 +175,22 @@ _int4_ws = {}
 
 
 def int4_workspace(device, nbytes: int) -> torch.Tensor:
-    """A per-device scratch tensor of at least ``nbytes`` for expanded int4 weights,
-    grown on demand and shared by every layer (launches on one stream run in order,
-    and its contents only live for the duration of one GEMM launch)."""
+    """A per-device scratch tensor of at least ``nbytes`` for ``gemm``'s ``workspace``
+    (expanded int4 weights, or the parked partial sums of int8 ranges), grown on demand
+    and shared by every layer (launches on one stream run in order, and its contents
+    only live for the duration of one GEMM launch)."""
     key = torch.device(device)
     ws = _int4_ws.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=key)
         _int4_ws[key] = ws
     return ws
+
+
+def park_bytes(m: int, n: int) -> int:
+    """Workspace that lets int8 codes with several ranges run on every tile size
+    (one fp32 tile per workgroup; the largest tile is 288 wide)."""
+    return 4 * (m + 288) * (n + 288)
 
 
 def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
@@ -196,7 +203,8 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
     accumulators (int32 for integer codes, float32 for e4m3).  ``workspace``: a
-    byte tensor the library may expand int4 weights into (see ``int4_workspace``).
+    byte tensor the library may expand int4 weights into, or park the sums of
+    finished int8 ranges in (see ``int4_workspace``, ``park_bytes``).
     """
     _need_cuda(a, b, a_neg, bias)
     raw = out_dtype == "acc"

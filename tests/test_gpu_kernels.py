@@ -352,6 +352,44 @@ def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
     assert (y0 - y1).abs().max().item() <= 2e-6 * y0.abs().max().item()
 
 
+@pytest.mark.parametrize("tile", [0, 11, 12, 13, 14, 15, 16])
+def test_gemm_int8_ranges_parked_in_a_lent_workspace(ops, tile):
+    """int8 with K segments and a two-tensor DualScale segment on every 8-wave tile: the sums of
+    finished ranges wait in the caller's workspace instead of a second register set.  Checked
+    against the closed form (fp64) and the second-accumulator kernels, ragged M and N, per-tensor
+    / per-token scales mixed, twice in a row on the same workspace; a workspace that is too small
+    is not used (same result as without)."""
+    M, N, K0, K1 = 333, 500, 256, 384
+    K = K0 + K1
+    a, a2 = _rand_codes((M, K), O.FMT_INT8, 51), _rand_codes((M, K), O.FMT_INT8, 52)
+    b = _rand_codes((N, K), O.FMT_INT8, 53)
+    ad, a2d, bd = (_to_dev_codes(t, O.FMT_INT8) for t in (a, a2, b))
+    g = torch.Generator().manual_seed(54)
+    s0 = torch.rand(1, generator=g) + 0.5
+    sx, sx2 = torch.rand(M, generator=g) + 0.5, torch.rand(M, generator=g) + 0.5
+    sw, bias = torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    rg = [ops.Range(0, K0, s0.to(DEV), sw.to(DEV), 0, 0, 1), ops.Range(K0, K1, sx.to(DEV), sw.to(DEV), 0, 1, 1),
+          ops.Range(K0, K1, sx2.to(DEV), sw.to(DEV), 1, 1, 1)]
+    kw = dict(m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT8, lda=K, ldb=K, bias=bias.to(DEV), a_neg=a2d)
+    swn = sw.numpy().astype(np.float64)[None, :]
+    want = (O.gemm_acc(a[:, :K0], b[:, :K0], O.FMT_INT8, O.FMT_INT8) / (float(s0) * swn) +
+            O.gemm_acc(a[:, K0:], b[:, K0:], O.FMT_INT8, O.FMT_INT8) / (sx.numpy().astype(np.float64)[:, None] * swn) +
+            O.gemm_acc(a2[:, K0:], b[:, K0:], O.FMT_INT8, O.FMT_INT8) / (sx2.numpy().astype(np.float64)[:, None] * swn) +
+            bias.numpy().astype(np.float64))
+    ws = torch.empty(ops.park_bytes(M, N), dtype=torch.uint8, device=DEV)
+    out = ops.gemm(ad, bd, rg, out_dtype=torch.float32, workspace=ws, tile=tile, **kw)
+    assert np.abs(_np(out).astype(np.float64) - want).max() <= 3e-6 * np.abs(want).max()
+    again = ops.gemm(ad, bd, rg, out_dtype=torch.float32, workspace=ws, tile=tile, **kw)
+    assert torch.equal(out, again)
+    if tile in (0, 12, 13, 14):  # tiles the second-accumulator kernels exist for
+        plain = ops.gemm(ad, bd, rg, out_dtype=torch.float32, tile=tile, **kw)
+        assert (out - plain).abs().max().item() <= 2e-6 * plain.abs().max().item()
+        small = ops.gemm(ad, bd, rg, out_dtype=torch.float32, workspace=ws[:4096], tile=tile, **kw)
+        assert torch.equal(small, plain)
+    o16 = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, workspace=ws, tile=tile, **kw)
+    assert (np.abs(_np(o16).astype(np.float64) - want) <= _bf16_ulp(want) + 1e-5 * np.abs(want).max()).all()
+
+
 @pytest.mark.parametrize("op", ["gelu_tanh", "gelu", "silu"])
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("dt", ["bf16", "fp32", "fp16"])
