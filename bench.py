@@ -22,6 +22,14 @@ PEAK_HBM = 8000.0                               # GB/s
 # HBM-side bytes per GEMM launch (fetched + written), from the two rocprofv3 --pmc runs
 # summarised in profiles/gemm_pipe_int8_flux_m4608.md (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB,
 # factors from a 256 MiB copy).  Counters cannot be read from inside this process.
+# the GEMM kernels the tile heuristic picks for each configuration's linears (rocprofv3 traces, profiles/)
+GEMM_KERNELS = {
+    1: "segq::gemm_kernel (int8, general)",
+    2: "segq::gemm_pipe_kernel<192,288> / <256,128, two ranges> (e4m3)",
+    3: "segq::gemm_pipe_kernel<192,288> / <288,192> (int8)",
+    4: "segq::gemm_pipe_kernel<128,128, group factors> (int8 x int4 expanded to int8)",
+    5: "segq::gemm_pipe_kernel<288,192> / <128,128> (int8 with parked ranges, e4m3 rescaled in place)",
+}
 MEASURED_TRAFFIC_BYTES = {3: 343.5e6}
 
 
@@ -165,7 +173,7 @@ def main():
         "config": {"workload": f"config {args.config}: " + ", ".join(f"{s.name} M{s.M} K{s.K} N{s.N} {s.kernel_type}" for s in specs),
                    "step": "activation quantize + segmented GEMM with fused dequant+bias, per linear",
                    "input_dtype": str(specs[0].x_dtype).replace("torch.", ""), "output_dtype": str(specs[0].x_dtype).replace("torch.", "")},
-        "roofline": {"bound": "mfma", "kernel": "segq::gemm_pipe_kernel<192,288> / <288,192> (int8)", "achieved": round(g_tops, 2), "peak": peak,
+        "roofline": {"bound": "mfma", "kernel": GEMM_KERNELS.get(args.config, "segq::gemm_pipe_kernel"), "achieved": round(g_tops, 2), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
                      "launches": n_g, "avg_launch_us": round(g_t / max(n_g, 1) * 1e6, 2),
                      "algorithmic_bytes_per_launch": round(g_bytes / max(n_g, 1)),

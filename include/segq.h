@@ -223,6 +223,14 @@ typedef struct segq_gemm_desc {
                          * The reference has per-tensor and per-row weight scales only
                          * (segquant/src/real_quant/real_gemm.cu:538-638); groups exist here alone. */
     int64_t group_dequant_stride; /* floats between consecutive groups, >= n */
+    int64_t split_k;    /* 0: the library decides; 1: never; s > 1: the K steps of every tile are shared by s
+                         * workgroups.  Splitting needs plain int8 or e4m3 codes, K ranges in multiples of 128,
+                         * batch == 1 and s * m * n * 4 bytes of workspace for the fp32 partial results (plus s
+                         * times the parking room above for int8 with several ranges); a second small kernel
+                         * sums them, adds the bias and rounds once.  For shapes with far fewer tiles than
+                         * compute units; no counterpart in the reference (its GemmUniversal runs one K
+                         * slice per problem: mode kGemm with batch_count 1,
+                         * segquant/src/real_quant/real_gemm.cu:281-285 and :424-445). */
     segq_krange ranges[SEGQ_MAX_RANGES];
 } segq_gemm_desc;
 

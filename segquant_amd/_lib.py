@@ -55,7 +55,7 @@ class GemmDesc(C.Structure):
         ("batch", C.c_int64), ("batch_stride_a", C.c_int64), ("batch_stride_b", C.c_int64),
         ("batch_stride_out", C.c_int64), ("batch_stride_sx", C.c_int64), ("batch_stride_sw", C.c_int64),
         ("n_ranges", C.c_int32), ("tile", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
-        ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64),
+        ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64), ("split_k", C.c_int64),
         ("ranges", KRange * SEGQ_MAX_RANGES),
     ]
 

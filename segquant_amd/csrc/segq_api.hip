@@ -83,6 +83,46 @@ __global__ void __launch_bounds__(256) expand_i4_kernel(const uint8_t* src, int6
     }
 }
 
+// Sum of the fp32 partial results of a split-K launch, plus bias, rounded once to the
+// output type.  VEC: four columns per thread.
+template <bool VEC>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* part, int splits, int64_t m, int64_t n, const void* bias,
+                                                            int bias_dtype, void* out, int out_dtype, int64_t ldo) {
+    constexpr int W = VEC ? 4 : 1;
+    const int64_t per_row = n / W;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= m * per_row) return;
+    const int64_t row = i / per_row, col = (i - row * per_row) * W;
+    float acc[W];
+#pragma unroll
+    for (int v = 0; v < W; ++v) acc[v] = 0.0f;
+    for (int z = 0; z < splits; ++z) {
+        const float* q = part + ((int64_t)z * m + row) * n + col;
+        if constexpr (VEC) {
+            const float4 t = *reinterpret_cast<const float4*>(q);
+            acc[0] += t.x; acc[1] += t.y; acc[2] += t.z; acc[3] += t.w;
+        } else {
+            acc[0] += q[0];
+        }
+    }
+    if (bias) {
+#pragma unroll
+        for (int v = 0; v < W; ++v) acc[v] += load_bias(bias, bias_dtype, col + v);
+    }
+    const int64_t e = row * ldo + col;
+    if (out_dtype == SEGQ_F32) {
+#pragma unroll
+        for (int v = 0; v < W; ++v) static_cast<float*>(out)[e + v] = acc[v];
+    } else if constexpr (VEC) {
+        const bool bf = out_dtype == SEGQ_BF16;
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + e) =
+            make_uint2(bf ? pack2_bf16(acc[0], acc[1]) : pack2_f16(acc[0], acc[1]), bf ? pack2_bf16(acc[2], acc[3]) : pack2_f16(acc[2], acc[3]));
+    } else {
+        const uint32_t two = out_dtype == SEGQ_BF16 ? pack2_bf16(acc[0], 0.0f) : pack2_f16(acc[0], 0.0f);
+        static_cast<uint16_t*>(out)[e] = (uint16_t)(two & 0xffffu);
+    }
+}
+
 static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     if (!d) return fail(SEGQ_ERR_ARG, "segq_gemm: null descriptor");
     if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
@@ -218,8 +258,59 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
-    if (d->tile != 0) park = park && park_fits(cfg);
-    if (park) p.park = static_cast<float*>(d->workspace);
+    // Split K: few tiles and a long contraction.  The K steps of every tile are shared by
+    // `splits` workgroups (grid.y), each writing an fp32 partial result into the workspace;
+    // a second kernel sums them, adds the bias and rounds.  Workspace: the partial results,
+    // then (int8 with several ranges) the parking slots of all those workgroups.
+    int splits = 1;
+    int64_t part_bytes = 0;
+    {
+        const bool can = plain8 && wide_ok && d->batch == 1 && !groups && d->out_dtype != SEGQ_ACC && d->workspace &&
+                         al(d->workspace, 16) && d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG);
+        const int64_t total_steps = ktotal / 128;
+        if (d->split_k > 1 && !can)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: split_k needs plain 8-bit codes, K ranges in multiples of 128, one problem, "
+                                              "a float output, an 8-wave tile and a workspace");
+        if (can) {
+            int want = 1, scfg = cfg;
+            const bool big_ok0 = !fold2 || park || f8;
+            if (d->split_k > 1) {
+                want = (int)(d->split_k < total_steps ? d->split_k : total_steps);
+                if (d->tile == 0) scfg = big_ok0 ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
+            } else if (d->tile == 0) {
+                const bool big_ok = !fold2 || park || f8;  // the 256 x 256 tile, or 256 x 128 with a second register set
+                scfg = big_ok ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
+                const TileCfg& t = TILE_CFGS[scfg];
+                const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
+                // measured: 48 tiles x 5 shares beat 192 tiles of 128 x 128 by 19 % (1024 x 15360 x 3072, e4m3),
+                // 96 tiles x 2 shares lose to 192 tiles of 256 x 128 (4096 x 6144 x 1536): the fp32 partial
+                // results and their sum cost what two shares gain
+                // (int8 with several ranges gains nothing: 139 -> 145 us on the same shape)
+                if (tiles * 4 <= 256 && total_steps >= 32 && !(i8 && fold)) {
+                    const int64_t by_cus = 256 / tiles, by_steps = total_steps / 8;
+                    want = (int)(by_cus < by_steps ? by_cus : by_steps);
+                    if (want > 16) want = 16;
+                }
+            }
+            const TileCfg& t = TILE_CFGS[scfg];
+            const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
+            const bool need_park = i8 && fold && scfg != FIRST_WIDE_CFG + 1 && scfg != FIRST_WIDE_CFG + 2 && scfg != FIRST_WIDE_CFG + 3;
+            auto bytes_for = [&](int s_) {
+                const int64_t pb = (((int64_t)s_ * d->m * d->n * 4) + 255) & ~(int64_t)255;
+                return pb + (need_park || park ? (int64_t)s_ * tiles * t.bm * t.bn * 4 : 0);
+            };
+            while (want > 1 && bytes_for(want) > d->workspace_bytes) --want;
+            if (d->split_k > 1 && want < 2) return fail(SEGQ_ERR_ARG, "segq_gemm: workspace too small for split_k");
+            if (want > 1) {
+                splits = want;
+                cfg = scfg;
+                part_bytes = (((int64_t)splits * d->m * d->n * 4) + 255) & ~(int64_t)255;
+                park = (need_park || park) && i8 && fold;
+            }
+        }
+    }
+    if (splits == 1 && d->tile != 0) park = park && park_fits(cfg);
+    if (park) p.park = reinterpret_cast<float*>(static_cast<uint8_t*>(d->workspace) + part_bytes);
     if (park) {
         // every 8-wave tile serves several ranges this way
     } else if (cfg >= FIRST_WIDE_CFG) {
@@ -241,6 +332,29 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
     p.vec_store = ((d->ldo * osz) % (4 * osz) == 0) && ((d->batch_stride_out * osz) % (4 * osz) == 0) && al(d->out, 4 * osz);
     p.vec_store16 = osz == 2 && d->ldo % 8 == 0 && d->batch_stride_out % 8 == 0 && al(d->out, 16);
+    if (splits > 1) {
+        p.splits = splits;
+        p.C = d->workspace;
+        p.ldc = d->n;
+        p.bsC = d->m * d->n;
+        p.bsA = p.bsB = p.bsSx = p.bsSw = 0;
+        p.out_dtype = SEGQ_F32;
+        p.bias = nullptr;
+        p.vec_store = d->n % 4 == 0;
+        p.vec_store16 = 0;
+        const int rc = i8 ? launch_gemm_i8(p, cfg, fold, splits, st) : launch_gemm_f8(p, cfg, fold, splits, st);
+        if (rc != SEGQ_OK) return rc;
+        const bool vec = d->n % 4 == 0 && d->ldo % 4 == 0 && al(d->out, 16);
+        const int64_t items = d->m * (vec ? d->n / 4 : d->n);
+        const dim3 grid((unsigned)((items + 255) / 256));
+        if (vec)
+            hipLaunchKernelGGL(splitk_reduce_kernel<true>, grid, dim3(256), 0, st, static_cast<const float*>(d->workspace), splits,
+                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo);
+        else
+            hipLaunchKernelGGL(splitk_reduce_kernel<false>, grid, dim3(256), 0, st, static_cast<const float*>(d->workspace), splits,
+                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo);
+        return check_launch("segq_gemm (split-K sum)");
+    }
     if (i8) return launch_gemm_i8(p, cfg, fold, d->batch, st);
     if (f8) return launch_gemm_f8(p, cfg, fold, d->batch, st);
     return launch_gemm_w4(p, cfg, fold, d->batch, st);

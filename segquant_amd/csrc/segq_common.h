@@ -43,6 +43,12 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 // Two fp32 values rounded to nearest even and packed, a in the low half
 // (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 on gfx950).
+__device__ __forceinline__ float load_bias(const void* bias, int dtype, int64_t n) {
+    if (dtype == SEGQ_F32) return static_cast<const float*>(bias)[n];
+    const uint32_t h = static_cast<const uint16_t*>(bias)[n];
+    return dtype == SEGQ_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+}
+
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t));
 }

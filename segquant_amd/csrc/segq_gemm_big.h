@@ -34,12 +34,6 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* g, uint8_t* lds_bas
     __builtin_amdgcn_global_load_lds((glb_ptr_t)g, (lds_ptr_t)lds_base, 16, 0, 0);
 }
 
-__device__ __forceinline__ float load_bias(const void* bias, int dtype, int n) {
-    if (dtype == SEGQ_F32) return static_cast<const float*>(bias)[n];
-    const uint32_t h = static_cast<const uint16_t*>(bias)[n];
-    return dtype == SEGQ_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
-}
-
 // Four consecutive outputs of one row, rounded once to the output type.
 template <int OUT>
 __device__ __forceinline__ void store4(void* C, int64_t e, const float (&o)[4], bool vec, int n_left) {

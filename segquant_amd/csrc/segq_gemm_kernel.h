@@ -46,6 +46,8 @@ struct GemmParams {
     int32_t tiles_m, tiles_n, group_m;
     int32_t vec_store;    // output rows allow 4-element vector stores
     int32_t vec_store16;  // 16-bit output rows allow 16-byte stores
+    int32_t splits;       // > 1: grid.y workgroups share the K steps of a tile (gemm_pipe_kernel only)
+    int32_t pad_;
     float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
     const float* grw;     // group-wise de-quantisation factors [K / 128][grw_gs], or null
     int64_t grw_gs;

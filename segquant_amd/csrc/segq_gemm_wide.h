@@ -471,6 +471,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     constexpr bool ACCF = FOLD && !F8 && !GRP && !PARK;
     constexpr bool HASF = ACCF || GRP;
     const acc_t acc_zero = {0, 0, 0, 0};
+    // Split K (p.splits > 1): workgroup (tile, y) multiplies the y-th share of the K steps,
+    // counted through the ranges, and writes an fp32 partial result that a second kernel
+    // sums.  r_last is the range its last step lies in: the one whose units its
+    // accumulators end up in (without a split: the last range).
+    int r_last = p.nr - 1, r_begin = 0;  // (r_begin: the range its first step lies in)
 
     static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
     static_assert(!F8 || (NS == 2 && TN >= 3), "the e4m3 schedule reads two weight fragments ahead in a two-stage ring");
@@ -608,11 +613,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             }
         }
     };
-    v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + (int64_t)blockIdx.x * (BM * BN / 4) + tid : nullptr;
+    v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (BM * BN / 4) + tid : nullptr;
     auto park = [&](int r) __attribute__((always_inline)) {
         if constexpr (PARK) {
-            if (r + 1 < p.nr) {
-                const int rl = p.nr - 1;
+            if (r < r_last) {
+                const int rl = r_last;
                 const float* sx = p.r[r].sx;
                 const float* sw = p.r[r].sw;
                 const float* sx2 = p.r[rl].sx;
@@ -633,14 +638,14 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                         fw[v] = sw2[n * cs2] * __builtin_amdgcn_rcpf(sw[n * cs]);
                     }
                     v4f old[TM];
-                    if (r > 0) {
+                    if (r > r_begin) {
 #pragma unroll
                         for (int b = 0; b < TM; ++b) old[b] = slot[(a * TM + b) * NT];
                     }
 #pragma unroll
                     for (int b = 0; b < TM; ++b) {
                         v4f t = __builtin_convertvector(acc[a][b], v4f) * (fw * fx[b]);
-                        if (r > 0) t += old[b];
+                        if (r > r_begin) t += old[b];
                         slot[(a * TM + b) * NT] = t;
                         acc[a][b] = acc_zero;
                     }
@@ -651,7 +656,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     auto fold = [&](int r) __attribute__((always_inline)) {
         if constexpr (FOLD && (F8 || GRP)) {
             auto& facc = [&]() -> auto& { if constexpr (GRP) return accf; else return acc; }();
-            if (r + 1 < p.nr) {  // rescale to the next range's units
+            if (r < r_last) {  // rescale to the next range's units
                 const float* sx = p.r[r].sx + z * p.bsSx;
                 const float* sw = p.r[r].sw + z * p.bsSw;
                 const float* sx2 = p.r[r + 1].sx + z * p.bsSx;
@@ -702,8 +707,23 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // (cr, ck) the tile being multiplied.  The end of the current range and the
     // source of its activations stay in registers, so the range table is read
     // only when a cursor crosses into the next range.
-    int lr = 0, lk = p.r[0].k0, lk1 = p.r[0].k1;
-    const uint8_t* la = (p.r[0].a_sel == 1) ? A2b : Ab;
+    int steps = 0;
+    for (int i = 0; i < p.nr; ++i) steps += (p.r[i].k1 - p.r[i].k0) / BK;
+    int lr = 0, skip = 0;  // this workgroup's first step: `skip` steps into range lr
+    if (p.splits > 1) {
+        skip = (int)((int64_t)steps * (int)blockIdx.y / p.splits);
+        steps = (int)((int64_t)steps * ((int)blockIdx.y + 1) / p.splits) - skip;
+        while (lr + 1 < p.nr && skip >= (p.r[lr].k1 - p.r[lr].k0) / BK) {
+            skip -= (p.r[lr].k1 - p.r[lr].k0) / BK;
+            ++lr;
+        }
+        r_last = r_begin = lr;
+        for (int left = skip + steps; r_last + 1 < p.nr && left > (p.r[r_last].k1 - p.r[r_last].k0) / BK; ++r_last)
+            left -= (p.r[r_last].k1 - p.r[r_last].k0) / BK;
+    }
+    const int r_first = lr, k_first = p.r[lr].k0 + skip * BK;
+    int lk = k_first, lk1 = p.r[lr].k1;
+    const uint8_t* la = (p.r[lr].a_sel == 1) ? A2b : Ab;
     auto advance_load = [&]() {
         lk += BK;
         if (lk >= lk1) {
@@ -714,8 +734,6 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             la = (p.r[rr].a_sel == 1) ? A2b : Ab;
         }
     };
-    int steps = 0;
-    for (int i = 0; i < p.nr; ++i) steps += (p.r[i].k1 - p.r[i].k0) / BK;
 
     // The epilogue's vectors (1/sx per row, 1/sw and bias per column of this tile)
     // are fetched first of all, so that the wait for the first DMA covers them, and
@@ -738,7 +756,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             lslot = (lslot + 1) & 3;
         }
     };
-    const int r_epi = ACCF ? 0 : p.nr - 1;  // the range whose units the accumulators end up in
+    const int r_epi = ACCF ? 0 : r_last;  // the range whose units the accumulators end up in
     float epi_val[EPI_IT];
     const bool want_epi = p.out_dtype != SEGQ_ACC;  // raw accumulators come with no scales at all (null pointers)
 #pragma unroll
@@ -789,7 +807,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // pipe of the whole SIMD (both its waves are in the same phase).  Issued one
     // at a time they never queue.  DMA_ and MORE_ are compile-time so that the
     // steady-state loop body has no branches.
-    int cr = 0, ck = p.r[0].k0, ck1 = p.r[0].k1;  // the tile being multiplied
+    int cr = r_first, ck = k_first, ck1 = p.r[r_first].k1;  // the tile being multiplied
+    bool dirty = false;  // int32 sums not yet folded into the fp32 set (a split can end inside a range)
     int buf = 0;                                   // its buffer, s % NS
     constexpr int NMF = TM * TN, NRD = TM + TN, NDM = A_IT + B_IT;
     constexpr int RD_EVERY = (NMF >= 2 * NRD + 4) ? 2 : 1;
@@ -915,10 +934,12 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         ck += BK;
         pslot = cslot;
         cslot = (cslot + 1) & 3;
+        dirty = true;
         if (ck >= ck1) {  // the range is complete: fold it, move to the next one
             if constexpr (GRP && FOLD) add_groups(acc, grw, pslot);  // this step's sums are still in the old range's units
             if constexpr (PARK) park(cr);
             else if constexpr (FOLD) fold(cr);
+            dirty = false;
             ++cr;
             const int rr = min(cr, p.nr - 1);
             ck = p.r[rr].k0;
@@ -934,6 +955,9 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (; s + NS < steps; ++s) step(std::true_type{}, std::true_type{});
     for (; s + 1 < steps; ++s) step(std::false_type{}, std::true_type{});
     if (s < steps) step(std::false_type{}, std::false_type{});
+    if constexpr (ACCF) {
+        if (dirty) fold(cr);
+    }
     if constexpr (GRP) {
         add_groups(acc, grw, pslot);  // the last step's sums
         v4f none[1][1];
@@ -942,13 +966,14 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         // the earlier ranges' sums come back in two halves, each with all its loads in flight at once
         v4f accp[TN][TM];
         constexpr int H = (TN + 1) / 2;
+        const bool parked = r_begin < r_last;  // (a split's share can lie inside one range)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             v4f old[H][TM];
 #pragma unroll
             for (int a = h * H; a < min(TN, (h + 1) * H); ++a)
 #pragma unroll
-                for (int b = 0; b < TM; ++b) old[a - h * H][b] = slot[(a * TM + b) * NT];
+                for (int b = 0; b < TM; ++b) old[a - h * H][b] = parked ? slot[(a * TM + b) * NT] : v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int a = h * H; a < min(TN, (h + 1) * H); ++a)
 #pragma unroll

@@ -193,12 +193,28 @@ def park_bytes(m: int, n: int) -> int:
     return 4 * (m + 288) * (n + 288)
 
 
+def split_bytes(m: int, n: int, splits: int = 16, park: bool = False) -> int:
+    """Workspace for a GEMM whose K steps are shared by up to ``splits`` workgroups per
+    tile: the fp32 partial results and, for int8 with several ranges (``park``), the
+    parking room of all those workgroups."""
+    return splits * (4 * m * n + (park_bytes(m, n) if park else 0)) + 256
+
+
+def auto_splits(m: int, n: int, k_steps: int) -> int:
+    """How many shares the library's own rule would take for an (m, n) problem of
+    ``k_steps`` 128-byte K steps (0: it would not split), to size the workspace with."""
+    tiles = -(-m // 256) * -(-n // 256)
+    if tiles * 4 > 256 or k_steps < 32:
+        return 0
+    return max(0, min(256 // tiles, k_steps // 8, 16))
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
          out_dtype, lda: int, ldb: int, a_neg: Optional[torch.Tensor] = None,
          bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
          tile: int = 0, workspace: Optional[torch.Tensor] = None,
-         group_dequant: Optional[torch.Tensor] = None) -> torch.Tensor:
+         group_dequant: Optional[torch.Tensor] = None, split_k: int = 0) -> torch.Tensor:
     """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
@@ -229,7 +245,7 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
     d.batch_stride_out = m * n; d.batch_stride_sx = batch_stride_sx; d.batch_stride_sw = batch_stride_sw
     if not 1 <= len(ranges) <= L.SEGQ_MAX_RANGES:
         raise RuntimeError(f"1..{L.SEGQ_MAX_RANGES} ranges")
-    d.n_ranges = len(ranges); d.tile = tile
+    d.n_ranges = len(ranges); d.tile = tile; d.split_k = split_k
     if workspace is not None:
         _need_cuda(workspace)
         d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()

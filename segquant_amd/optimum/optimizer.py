@@ -326,6 +326,12 @@ class DefaultOptimizer(BaseOptimizer):
         # 441 -> 383 us; 9216 tokens: 1044 -> 756 us; no gain at 1024 tokens)
         if ws is None and gdq is None and plan["fa"] == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1 and M >= 2048:
             ws = ops.int4_workspace(x.device, ops.park_bytes(M, N))
+        # few tiles, long K (config 5 at 1024 tokens): room for the library to share the K steps of a
+        # tile between workgroups (it does for e4m3 and for single-range int8)
+        if ws is None and gdq is None and plan["fw"] != ops.FMT_INT4:
+            ns = ops.auto_splits(M, N, sum(r.k_len for r in ranges) // 128)
+            if ns > 1:
+                ws = ops.int4_workspace(x.device, ops.split_bytes(M, N, ns))
         out = ops.gemm(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
                        lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws, group_dequant=gdq)
         return out.view(*x.shape[:-1], N)

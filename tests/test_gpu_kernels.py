@@ -352,6 +352,50 @@ def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
     assert (y0 - y1).abs().max().item() <= 2e-6 * y0.abs().max().item()
 
 
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("tile", [0, 11, 12, 14, 16])
+def test_gemm_split_k(ops, fmt, tile):
+    """The K steps of every tile shared by 2..7 workgroups, shares that begin and end inside
+    ranges, one range and three (K segments + a two-tensor DualScale segment), ragged M and N,
+    an N that allows no vector stores: equal to the unsplit launch up to fp32 summation order,
+    and to the closed form; what cannot be split is refused."""
+    M, N, K0, K1 = 210, 330, 384, 640
+    K = K0 + K1
+    a, a2, b = _rand_codes((M, K), fmt, 61), _rand_codes((M, K), fmt, 62), _rand_codes((N, K), fmt, 63)
+    ad, a2d, bd = (_to_dev_codes(t, fmt) for t in (a, a2, b))
+    g = torch.Generator().manual_seed(64)
+    s0 = torch.rand(1, generator=g) + 0.5
+    sx, sx2 = torch.rand(M, generator=g) + 0.5, torch.rand(M, generator=g) + 0.5
+    sw, bias = torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    one = [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
+    three = [ops.Range(0, K0, s0.to(DEV), sw.to(DEV), 0, 0, 1), ops.Range(K0, K1, sx.to(DEV), sw.to(DEV), 0, 1, 1),
+             ops.Range(K0, K1, sx2.to(DEV), sw.to(DEV), 1, 1, 1)]
+    ws = torch.empty(ops.split_bytes(M, N, 8, park=True), dtype=torch.uint8, device=DEV)
+    tol = 3e-6 if fmt == O.FMT_INT8 else 3e-4
+    for n_cols in (N, N - 1):  # N - 1: rows of the fp32 partial results are not 16-byte multiples
+        kw = dict(m=M, n=n_cols, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, bias=bias[:n_cols].contiguous().to(DEV), a_neg=a2d, tile=tile)
+        for rg in (one, three):
+            rg = [ops.Range(r.k_begin, r.k_len, r.sx, r.sw[:n_cols].contiguous(), r.a_sel, r.sx_row_stride, r.sw_col_stride) for r in rg]
+            ref = ops.gemm(ad, bd, rg, out_dtype=torch.float32, split_k=1, workspace=ws, **kw)
+            for sk in (2, 3, 7):
+                out = ops.gemm(ad, bd, rg, out_dtype=torch.float32, split_k=sk, workspace=ws, **kw)
+                assert (out - ref).abs().max().item() <= tol * ref.abs().max().item(), (n_cols, len(rg), sk)
+            o16 = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, split_k=3, workspace=ws, **kw)
+            r16 = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, split_k=1, workspace=ws, **kw)
+            assert (o16.float() - r16.float()).abs().max().item() <= 2.0 ** -7 * r16.float().abs().max().item()
+    av, a2v, bv = (O.code_values(t, fmt) for t in (a, a2, b))
+    swn = sw.numpy().astype(np.float64)[None, :]
+    want = (av[:, :K0] @ bv[:, :K0].T / (float(s0) * swn) + av[:, K0:] @ bv[:, K0:].T / (sx.numpy().astype(np.float64)[:, None] * swn) +
+            a2v[:, K0:] @ bv[:, K0:].T / (sx2.numpy().astype(np.float64)[:, None] * swn) + bias.numpy().astype(np.float64))
+    out = ops.gemm(ad, bd, three, out_dtype=torch.float32, split_k=5, workspace=ws, m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K,
+                   bias=bias.to(DEV), a_neg=a2d, tile=tile)
+    assert np.abs(_np(out).astype(np.float64) - want).max() <= (5e-6 if fmt == O.FMT_INT8 else 1e-3) * np.abs(want).max()
+    with pytest.raises(RuntimeError):  # no workspace
+        ops.gemm(ad, bd, one, out_dtype=torch.float32, split_k=2, m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K)
+    with pytest.raises(RuntimeError):  # the general kernels do not split
+        ops.gemm(ad, bd, one, out_dtype=torch.float32, split_k=2, workspace=ws, tile=3, m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K)
+
+
 @pytest.mark.parametrize("tile", [0, 11, 12, 13, 14, 15, 16])
 def test_gemm_int8_ranges_parked_in_a_lent_workspace(ops, tile):
     """int8 with K segments and a two-tensor DualScale segment on every 8-wave tile: the sums of
