@@ -128,6 +128,11 @@ typedef struct segq_quant_desc {
     int32_t pre_op;     /* segq_pre_op */
     const void* gate;   /* device or NULL: rows x cols of x_dtype, row stride ld_gate; needs a pre_op */
     int64_t ld_gate;
+    const float* col_div; /* device or NULL: cols divisors, 16-byte aligned.  Every element (after the pre_op, if
+                         * any) is divided by the divisor of its column and the quotient rounded to x_dtype: the
+                         * SmoothQuant step x / s that the reference applies to a clone of the activation right
+                         * before it quantises it (segquant/optimum/optimizer.py:467-470, :517).  Pass s as the
+                         * reference uses it, i.e. already rounded to x_dtype. */
 } segq_quant_desc;
 
 int segq_quantize(const segq_quant_desc* d, segq_stream_t stream);
@@ -223,6 +228,11 @@ typedef struct segq_gemm_desc {
                          * The reference has per-tensor and per-row weight scales only
                          * (segquant/src/real_quant/real_gemm.cu:538-638); groups exist here alone. */
     int64_t group_dequant_stride; /* floats between consecutive groups, >= n */
+    const void* addend; /* device or NULL: (m, n) values of out_dtype, row stride ld_addend, batch stride
+                         * batch_stride_out, added to the result before its one rounding (a residual, or the
+                         * low-rank branch x L1 L2 that the reference's SVD optimiser adds to the quantised
+                         * product as a separate operator, segquant/optimum/optimizer.py:731-740) */
+    int64_t ld_addend;
     int64_t split_k;    /* 0: the library decides; 1: never; s > 1: the K steps of every tile are shared by s
                          * workgroups.  Splitting needs plain int8 or e4m3 codes, K ranges in multiples of 128,
                          * batch == 1 and s * m * n * 4 bytes of workspace for the fp32 partial results (plus s

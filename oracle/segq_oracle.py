@@ -325,6 +325,16 @@ def activation(x, op: str, gate=None, dtype: str = "fp32") -> np.ndarray:
     return round_to_dtype((_f32(x) * f(gate)).astype(np.float32), dtype)
 
 
+def smooth_divide(x, s, dtype: str = "fp32") -> np.ndarray:
+    """SmoothQuant's activation step ``x.div_(s.to(x.dtype))``
+    (segquant/optimum/optimizer.py:467-470): an fp32 division by the divisor rounded
+    to the tensor's dtype, the quotient rounded to that dtype; ``s`` has one entry per
+    column.  IEEE division is correctly rounded everywhere, so torch's CPU result pins
+    this bit for bit."""
+    sd = round_to_dtype(_f32(s).reshape(1, -1), dtype)
+    return round_to_dtype((_f32(x) / sd).astype(np.float32), dtype)
+
+
 def group_amax(w, group: int) -> np.ndarray:
     """|w| maxima over runs of ``group`` input channels: (N, K) -> (N, K / group).
     Group-wise weight scales are not in the reference (its weight scales are per

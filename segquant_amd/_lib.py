@@ -32,7 +32,7 @@ class QuantDesc(C.Structure):
         ("kseg_stride", C.c_int64),
         ("n_kseg", C.c_int32), ("dual", C.c_int32), ("dual_kseg_mask", C.c_uint32), ("dynamic", C.c_int32),
         ("kseg_bounds", C.c_int64 * (SEGQ_MAX_KSEG + 1)),
-        ("pre_op", C.c_int32), ("gate", C.c_void_p), ("ld_gate", C.c_int64),
+        ("pre_op", C.c_int32), ("gate", C.c_void_p), ("ld_gate", C.c_int64), ("col_div", C.c_void_p),
     ]
 
 
@@ -55,7 +55,8 @@ class GemmDesc(C.Structure):
         ("batch", C.c_int64), ("batch_stride_a", C.c_int64), ("batch_stride_b", C.c_int64),
         ("batch_stride_out", C.c_int64), ("batch_stride_sx", C.c_int64), ("batch_stride_sw", C.c_int64),
         ("n_ranges", C.c_int32), ("tile", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
-        ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64), ("split_k", C.c_int64),
+        ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64),
+        ("addend", C.c_void_p), ("ld_addend", C.c_int64), ("split_k", C.c_int64),
         ("ranges", KRange * SEGQ_MAX_RANGES),
     ]
 

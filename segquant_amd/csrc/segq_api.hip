@@ -87,7 +87,8 @@ __global__ void __launch_bounds__(256) expand_i4_kernel(const uint8_t* src, int6
 // output type.  VEC: four columns per thread.
 template <bool VEC>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* part, int splits, int64_t m, int64_t n, const void* bias,
-                                                            int bias_dtype, void* out, int out_dtype, int64_t ldo) {
+                                                            int bias_dtype, void* out, int out_dtype, int64_t ldo,
+                                                            const void* addend, int64_t ldadd) {
     constexpr int W = VEC ? 4 : 1;
     const int64_t per_row = n / W;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -108,6 +109,11 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* part, i
     if (bias) {
 #pragma unroll
         for (int v = 0; v < W; ++v) acc[v] += load_bias(bias, bias_dtype, col + v);
+    }
+    if (addend) {  // same dtype as the output
+        const int64_t ea = row * ldadd + col;
+#pragma unroll
+        for (int v = 0; v < W; ++v) acc[v] += load_bias(addend, out_dtype, ea + v);
     }
     const int64_t e = row * ldo + col;
     if (out_dtype == SEGQ_F32) {
@@ -141,6 +147,8 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         d->batch_stride_a % 16 || d->batch_stride_b % 16)
         return fail(SEGQ_ERR_ARG, "segq_gemm: a and b need 16-byte aligned bases and row strides");
     if (d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
+    if (d->addend && (d->out_dtype == SEGQ_ACC || d->ld_addend < d->n))
+        return fail(SEGQ_ERR_ARG, "segq_gemm: an addend needs a float output and ld_addend >= n");
     const bool groups = d->group_dequant != nullptr;
     if (groups) {
         if (!(i8 || w4) || d->batch != 1 || d->out_dtype == SEGQ_ACC || d->group_dequant_stride < d->n || !al(d->group_dequant, 4))
@@ -221,6 +229,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     p.bsA = d->batch_stride_a; p.bsB = d->batch_stride_b; p.bsC = d->batch_stride_out;
     p.bsSx = d->batch_stride_sx; p.bsSw = d->batch_stride_sw;
     p.out_dtype = d->out_dtype; p.bias_dtype = d->bias_dtype;
+    {
+        const int64_t asz = d->out_dtype == SEGQ_F32 ? 4 : 2;
+        p.addend = d->addend;
+        p.ldadd = d->ld_addend;
+        p.vec_add = d->addend && (d->ld_addend * asz) % (4 * asz) == 0 && (d->batch_stride_out * asz) % (4 * asz) == 0 && al(d->addend, 4 * asz);
+    }
     p.nr = d->n_ranges;
     const bool fold = d->n_ranges > 1;
     bool wide_ok = d->m * d->lda < (int64_t)1 << 32 && d->n * d->ldb < (int64_t)1 << 32;
@@ -340,6 +354,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         p.bsA = p.bsB = p.bsSx = p.bsSw = 0;
         p.out_dtype = SEGQ_F32;
         p.bias = nullptr;
+        p.addend = nullptr;
         p.vec_store = d->n % 4 == 0;
         p.vec_store16 = 0;
         const int rc = i8 ? launch_gemm_i8(p, cfg, fold, splits, st) : launch_gemm_f8(p, cfg, fold, splits, st);
@@ -349,10 +364,10 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         const dim3 grid((unsigned)((items + 255) / 256));
         if (vec)
             hipLaunchKernelGGL(splitk_reduce_kernel<true>, grid, dim3(256), 0, st, static_cast<const float*>(d->workspace), splits,
-                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo);
+                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo, d->addend, d->ld_addend);
         else
             hipLaunchKernelGGL(splitk_reduce_kernel<false>, grid, dim3(256), 0, st, static_cast<const float*>(d->workspace), splits,
-                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo);
+                               d->m, d->n, d->bias, d->bias_dtype, d->out, d->out_dtype, d->ldo, d->addend, d->ld_addend);
         return check_launch("segq_gemm (split-K sum)");
     }
     if (i8) return launch_gemm_i8(p, cfg, fold, d->batch, st);

@@ -281,6 +281,7 @@ __global__ void __launch_bounds__(256) gemm_big_kernel(const GemmParams p) {
                             float o[4];
 #pragma unroll
                             for (int v = 0; v < 4; ++v) o[v] = (float)acc[a][b][q * 4 + v] * rx[b] * rw[v] + bv[v];
+                            add_addend4(p, z, m, n, o);
                             store4<OUT>(p.C, e, o, vec, p.N - n);
                         }
                     }

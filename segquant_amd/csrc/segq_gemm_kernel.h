@@ -46,6 +46,10 @@ struct GemmParams {
     int32_t tiles_m, tiles_n, group_m;
     int32_t vec_store;    // output rows allow 4-element vector stores
     int32_t vec_store16;  // 16-bit output rows allow 16-byte stores
+    const void* addend;   // (M, N) tensor of the output's dtype added before the one rounding, or null
+    int64_t ldadd;
+    int32_t vec_add;      // its rows allow 4-element vector loads
+    int32_t pad2_;
     int32_t splits;       // > 1: grid.y workgroups share the K steps of a tile (gemm_pipe_kernel only)
     int32_t pad_;
     float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
@@ -55,6 +59,36 @@ struct GemmParams {
 };
 
 enum { GEMM_I8 = 0, GEMM_F8 = 1 };
+
+// o[0..3] += addend[z][m][n .. n + 3] (columns beyond N skipped)
+__device__ __forceinline__ void add_addend4(const GemmParams& p, int64_t z, int m, int n, float (&o)[4]) {
+    if (!p.addend) return;
+    const int64_t e = z * p.bsC + (int64_t)m * p.ldadd + n;
+    if (p.out_dtype == SEGQ_F32) {
+        const float* q = static_cast<const float*>(p.addend) + e;
+        if (p.vec_add && n + 3 < p.N) {
+            const float4 t = *reinterpret_cast<const float4*>(q);
+            o[0] += t.x; o[1] += t.y; o[2] += t.z; o[3] += t.w;
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < p.N) o[v] += q[v];
+        }
+    } else {
+        const uint16_t* q = static_cast<const uint16_t*>(p.addend) + e;
+        uint32_t h[4] = {0, 0, 0, 0};
+        if (p.vec_add && n + 3 < p.N) {
+            const uint2 t = *reinterpret_cast<const uint2*>(q);
+            h[0] = t.x & 0xffffu; h[1] = t.x >> 16; h[2] = t.y & 0xffffu; h[3] = t.y >> 16;
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < p.N) h[v] = q[v];
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) o[v] += (p.out_dtype == SEGQ_BF16) ? bf16_bits_to_f32(h[v]) : f16_bits_to_f32(h[v]);
+    }
+}
 constexpr int BK = 128;  // code bytes of K per step
 
 // Chunk swizzle.  The LDS of gfx950 has 64 banks of 4 bytes (a 256-byte span),
@@ -375,6 +409,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
                 if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
                 else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
             }
+            add_addend4(p, z, m, n, o);
             const int64_t e = c_off + (int64_t)m * p.ldc + n;
             const bool vec = p.vec_store && (n + 3 < p.N);
             if (p.out_dtype == SEGQ_F32) {

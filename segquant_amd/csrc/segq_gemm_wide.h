@@ -117,6 +117,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
                     o[v] = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
+                add_addend4(p, z, min(m_base + b * 16, p.M - 1), n_base + a * 16, o);
                 const bool bf = p.out_dtype == SEGQ_BF16;
                 *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
                     make_uint2(bf ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]),
@@ -130,8 +131,9 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
                 if ((16 * CH) % 64 != 0 && c >= 16 * CH) continue;
                 const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + col * 16);
                 const int m = m0 + wm * WM + b * 16 + row;
-                if (m < p.M)
+                if (m < p.M) {
                     *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + col * 8) = v;
+                }
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -156,6 +158,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
                 if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
                 else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
             }
+            add_addend4(p, z, m, n, o);
             const int64_t e = c_off + (int64_t)m * p.ldc + n;
             const bool vec = p.vec_store && (n + 3 < p.N);
             if (p.out_dtype == SEGQ_F32) store4<SEGQ_F32>(p.C, e, o, vec, p.N - n);

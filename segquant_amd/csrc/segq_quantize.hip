@@ -24,6 +24,7 @@ struct QuantParams {
     int32_t pre_op;   // segq_pre_op applied to the input before it is quantised
     const void* gate; // with a pre_op: x is multiplied by op(gate) instead of being replaced by op(x)
     int64_t ldg;
+    const float* col_div;  // per-column divisors (SmoothQuant's s), applied after the pre_op, or null
     int32_t kb[SEGQ_MAX_KSEG + 1];
 };
 
@@ -256,21 +257,37 @@ template <int DT>
 __device__ __forceinline__ void pre_run(const QuantParams& p, int64_t row, int64_t col, RawRun<DT>& r) {
     float v[16];
     raw_to_f32<DT>(r, v);
-    if (p.gate) {
-        const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
-        RawRun<DT> gr;
-        load_raw<DT>(static_cast<const uint8_t*>(p.gate) + (row * p.ldg + col) * esz, gr);
-        float g[16];
-        raw_to_f32<DT>(gr, g);
+    if (p.pre_op != SEGQ_PRE_NONE) {
+        if (p.gate) {
+            const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
+            RawRun<DT> gr;
+            load_raw<DT>(static_cast<const uint8_t*>(p.gate) + (row * p.ldg + col) * esz, gr);
+            float g[16];
+            raw_to_f32<DT>(gr, g);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) g[i] = act_value(p.pre_op, g[i]);
-        f32_to_raw<DT>(g, gr);
-        raw_to_f32<DT>(gr, g);
+            for (int i = 0; i < 16; ++i) g[i] = act_value(p.pre_op, g[i]);
+            f32_to_raw<DT>(g, gr);
+            raw_to_f32<DT>(gr, g);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] *= g[i];
-    } else {
+            for (int i = 0; i < 16; ++i) v[i] *= g[i];
+        } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = act_value(p.pre_op, v[i]);
+            for (int i = 0; i < 16; ++i) v[i] = act_value(p.pre_op, v[i]);
+        }
+        if (p.col_div) {  // the activation's result is rounded to the dtype before it is divided
+            f32_to_raw<DT>(v, r);
+            raw_to_f32<DT>(r, v);
+        }
+    }
+    if (p.col_div) {
+        // x / s as torch's in-place div_ in the tensor's dtype: an IEEE fp32 division, rounded to the dtype
+        const float4* q = reinterpret_cast<const float4*>(p.col_div + col);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 t = q[i];
+            v[4 * i + 0] = v[4 * i + 0] / t.x; v[4 * i + 1] = v[4 * i + 1] / t.y;
+            v[4 * i + 2] = v[4 * i + 2] / t.z; v[4 * i + 3] = v[4 * i + 3] / t.w;
+        }
     }
     f32_to_raw<DT>(v, r);
 }
@@ -521,9 +538,9 @@ static int launch_quant(const QuantParams& p, hipStream_t st) {
 template <int DT>
 static int launch_quant_fmt(const QuantParams& p, hipStream_t st) {
     switch (p.fmt) {
-        case SEGQ_CODE_I8: return p.pre_op ? launch_quant<DT, SEGQ_CODE_I8, true>(p, st) : launch_quant<DT, SEGQ_CODE_I8, false>(p, st);
-        case SEGQ_CODE_E4M3: return p.pre_op ? launch_quant<DT, SEGQ_CODE_E4M3, true>(p, st) : launch_quant<DT, SEGQ_CODE_E4M3, false>(p, st);
-        case SEGQ_CODE_I4: return p.pre_op ? launch_quant<DT, SEGQ_CODE_I4, true>(p, st) : launch_quant<DT, SEGQ_CODE_I4, false>(p, st);
+        case SEGQ_CODE_I8: return (p.pre_op || p.col_div) ? launch_quant<DT, SEGQ_CODE_I8, true>(p, st) : launch_quant<DT, SEGQ_CODE_I8, false>(p, st);
+        case SEGQ_CODE_E4M3: return (p.pre_op || p.col_div) ? launch_quant<DT, SEGQ_CODE_E4M3, true>(p, st) : launch_quant<DT, SEGQ_CODE_E4M3, false>(p, st);
+        case SEGQ_CODE_I4: return (p.pre_op || p.col_div) ? launch_quant<DT, SEGQ_CODE_I4, true>(p, st) : launch_quant<DT, SEGQ_CODE_I4, false>(p, st);
     }
     return fail(SEGQ_ERR_ARG, "segq_quantize: unknown code_fmt %d", p.fmt);
 }
@@ -571,6 +588,8 @@ int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_b
             return fail(SEGQ_ERR_ARG, "segq_quantize: gate must be 16-byte aligned with ld_gate >= cols");
     }
     p.pre_op = d->pre_op; p.gate = d->gate; p.ldg = d->ld_gate;
+    if (d->col_div && !aligned16(d->col_div)) return fail(SEGQ_ERR_ARG, "segq_quantize: col_div must be 16-byte aligned");
+    p.col_div = d->col_div;
     if (d->n_kseg == 1) {
         p.kb[0] = 0; p.kb[1] = (int32_t)d->cols;
     } else {

@@ -173,17 +173,25 @@ class SegmentLinear(nn.Module):
         fn = {"gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "gelu": F.gelu, "silu": F.silu}[pre_op]
         return fn(x) if gate is None else x * fn(gate)
 
-    def forward(self, x, chunked=False, pre_op=None, gate=None):
+    def forward(self, x, chunked=False, pre_op=None, gate=None, col_div=None, addend=None):
         """``pre_op`` ("gelu_tanh", "gelu", "silu") and ``gate`` are not in the reference: they
         hand the activation function of the module in front (x -> op(x), or x * op(gate) for
         GEGLU / SwiGLU, backend/torch/layers/activations.py:52-57, :77-80, :110-121) to this
         layer, whose quantise kernel evaluates it on the fly instead of reading back a stored
-        activation tensor.  The layer must have been calibrated on the activated input."""
+        activation tensor.  The layer must have been calibrated on the activated input.
+        ``col_div`` (per input channel, applied after the activation) and ``addend`` (added to
+        the output) are the hooks for the reference's SmoothQuant division and SVD low-rank
+        branch (segquant/optimum/optimizer.py:467-470, :731-740), fused into the same kernels."""
         opt = self.optimizer
         if not chunked and opt.real_quant and opt.has_calibrated:
-            return opt.forward_fused(x, self.bias_data if self.bias else None, pre_op=pre_op, gate=gate)
+            return opt.forward_fused(x, self.bias_data if self.bias else None, pre_op=pre_op, gate=gate,
+                                     col_div=col_div, addend=addend)
         if pre_op is not None:
             x = self._activated(x, pre_op, gate)
+        if col_div is not None:
+            x = x / col_div.to(x.dtype)
+        if addend is not None:
+            return self.forward(x, chunked=chunked) + addend
         if not chunked and not self.equal_chunks:
             res = opt.forward_fake(x)
             return res + self.bias_data if self.bias else res

@@ -105,7 +105,7 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
              dual: bool = False, dual_kseg_mask: int = 0xFFFFFFFF, dynamic: bool = False,
              two_tensors: bool = False, out: Optional[torch.Tensor] = None,
              out_neg: Optional[torch.Tensor] = None, pre_op: Optional[str] = None,
-             gate: Optional[torch.Tensor] = None):
+             gate: Optional[torch.Tensor] = None, col_div: Optional[torch.Tensor] = None):
     """Quantise a 2-D float matrix ``x`` (rows, cols) to codes.
 
     See ``segq_quantize`` in include/segq.h for the scale indexing.  Returns the
@@ -114,6 +114,9 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
     written by the kernel.  ``pre_op`` ("gelu_tanh", "gelu", "silu") fuses the
     activation function in front of the linear: op(x) is quantised, or
     x * op(gate) when ``gate`` (same shape and dtype as ``x``) is given.
+    ``col_div``: one divisor per column (SmoothQuant's ``s``, any float dtype; it is
+    used rounded to ``x.dtype`` as the reference's ``x.div_(s.to(x.dtype))`` does),
+    applied after the ``pre_op``.
     """
     _need_cuda(x, scale, scale_neg, gate)
     if x.dim() != 2 or x.stride(1) != 1:
@@ -146,6 +149,12 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
         if pre_op not in PRE_OPS:
             raise RuntimeError(f"pre_op must be one of {sorted(PRE_OPS)}")
         d.pre_op = PRE_OPS[pre_op]
+    if col_div is not None:
+        _need_cuda(col_div)
+        if col_div.numel() != cols:
+            raise RuntimeError("col_div needs one entry per column")
+        col_div = col_div.reshape(-1).to(x.dtype).to(torch.float32).contiguous()
+        d.col_div = col_div.data_ptr()
     if gate is not None:
         if pre_op is None or gate.shape != x.shape or gate.dtype != x.dtype or gate.stride(1) != 1:
             raise RuntimeError("gate needs a pre_op and the shape, dtype and contiguous rows of x")
@@ -214,7 +223,8 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
          bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
          tile: int = 0, workspace: Optional[torch.Tensor] = None,
-         group_dequant: Optional[torch.Tensor] = None, split_k: int = 0) -> torch.Tensor:
+         group_dequant: Optional[torch.Tensor] = None, split_k: int = 0,
+         addend: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
@@ -249,6 +259,11 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
     if workspace is not None:
         _need_cuda(workspace)
         d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()
+    if addend is not None:
+        _need_cuda(addend)
+        if raw or addend.dtype != tdt or addend.shape != out.shape or not addend.is_contiguous():
+            raise RuntimeError("addend must be a contiguous tensor of the output's shape and dtype")
+        d.addend = addend.data_ptr(); d.ld_addend = n
     if group_dequant is not None:
         _need_cuda(group_dequant)
         if group_dequant.dtype != torch.float32 or group_dequant.dim() != 2 or group_dequant.stride(1) != 1:

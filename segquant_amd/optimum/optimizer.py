@@ -253,7 +253,7 @@ class DefaultOptimizer(BaseOptimizer):
                           sw_cs=1 if sw_vec.numel() > 1 else 0, bounds=bounds, N=N, K=K)
         return self._plan
 
-    def forward_fused(self, x: torch.Tensor, bias=None, pre_op=None, gate=None) -> torch.Tensor:
+    def forward_fused(self, x: torch.Tensor, bias=None, pre_op=None, gate=None, col_div=None, addend=None) -> torch.Tensor:
         """Final (..., out) result in ``x.dtype``: quantise + segmented GEMM with
         de-quantisation and bias fused.  Equivalent to ``forward`` followed by
         the recombination of ``SegmentLinear.forward``, with the partial sums of
@@ -261,7 +261,12 @@ class DefaultOptimizer(BaseOptimizer):
 
         ``pre_op`` / ``gate``: the layer's input is op(x), or x * op(gate), with
         the activation function evaluated inside the quantise kernel (see
-        ``ops.quantize``); the scales must have been calibrated on that input."""
+        ``ops.quantize``); the scales must have been calibrated on that input.
+        ``col_div``: one divisor per input channel applied before quantising (the
+        reference's SmoothQuant step ``x / s``, optimizer.py:467-470; the weights must
+        have been multiplied by ``s``).  ``addend``: a (..., out) tensor of ``x.dtype``
+        added to the result before its one rounding (the SVD optimiser's low-rank
+        branch, optimizer.py:731-740)."""
         plan = self._plan or self._build_plan(x.device)
         K, N = plan["K"], plan["N"]
         x2 = x.reshape(-1, K)
@@ -302,7 +307,8 @@ class DefaultOptimizer(BaseOptimizer):
         # registers), measured on the 4608 x 15360 x 3072 shape.
         codes = ops.quantize(x2, plan["fa"], pos, neg, row_stride=1 if per_tok else 0,
                              kseg_bounds=bounds if S > 1 else None, kseg_stride=kstride, dual=dual,
-                             dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual, pre_op=pre_op, gate=gate)
+                             dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual, pre_op=pre_op, gate=gate,
+                             col_div=col_div)
         codes, codes_neg = codes if dual else (codes, None)
         ranges = []
         for s in range(S):
@@ -333,5 +339,6 @@ class DefaultOptimizer(BaseOptimizer):
             if ns > 1:
                 ws = ops.int4_workspace(x.device, ops.split_bytes(M, N, ns))
         out = ops.gemm(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
-                       lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws, group_dequant=gdq)
+                       lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws, group_dequant=gdq,
+                       addend=None if addend is None else addend.reshape(M, N).contiguous())
         return out.view(*x.shape[:-1], N)

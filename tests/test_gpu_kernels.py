@@ -482,6 +482,72 @@ def test_quantize_with_fused_activation(ops, op, gated, dt):
         assert (np.abs(v_got - v_want) <= 0.126 * np.abs(v_want) + 2.0 ** -9).all()  # neighbouring e4m3 values
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp32", "fp16"])
+def test_quantize_with_column_divisors(ops, dt):
+    """SmoothQuant's x / s inside the quantise kernel: bit-exact against the oracle (IEEE
+    division, no transcendental function involved), static and dynamic, alone and after a
+    fused activation (there to the fused activation's own bound)."""
+    tdt = TDT[dt]
+    rows, cols = 37, 1040
+    g = torch.Generator().manual_seed(45)
+    x = (torch.randn(rows, cols, generator=g) * 3).to(tdt)
+    sdiv = torch.rand(cols, generator=g) * 4 + 0.05
+    xd = x.to(DEV)
+    want = O.smooth_divide(x.float().numpy(), sdiv.numpy(), dt)
+    s = (torch.rand(rows, generator=g) * 20 + 0.5)
+    for fmt in FMTS:
+        c = ops.quantize(xd, fmt, s.to(DEV), row_stride=1, col_div=sdiv.to(DEV))
+        assert np.array_equal(_codes_np(c, fmt), O.quantize_act(want[None], s.numpy(), fmt)[0])
+    scale = torch.empty(rows, device=DEV)
+    c = ops.quantize(xd, O.FMT_INT8, scale, row_stride=1, dynamic=True, col_div=sdiv.to(DEV))
+    want_scale = O.row_scale_div(np.abs(want).max(axis=1), 127.0)
+    assert np.array_equal(scale.cpu().numpy(), want_scale)
+    assert np.array_equal(c.cpu().numpy(), O.quantize_act(want[None], want_scale, O.FMT_INT8)[0])
+    act = O.smooth_divide(O.activation(x.float().numpy(), "silu", dtype=dt), sdiv.numpy(), dt)
+    c = ops.quantize(xd, O.FMT_INT8, s.to(DEV), row_stride=1, col_div=sdiv.to(DEV), pre_op="silu")
+    d = np.abs(c.cpu().numpy().astype(np.int32) - O.quantize_act(act[None], s.numpy(), O.FMT_INT8)[0].astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() <= 4e-3
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3, O.FMT_INT4])
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_gemm_addend(ops, fmt, dt):
+    """out = acc / (sx sw) + bias + addend, rounded once: every kernel family (general, 8-wave
+    through LDS and direct, 32 x 32, split K), ragged shapes, a batch."""
+    M, N, K, Z = 150, 264, 256, 2
+    fa = O.FMT_INT8 if fmt == O.FMT_INT4 else fmt
+    a = np.stack([_rand_codes((M, K), fa, 70 + z) for z in range(Z)])
+    b = np.stack([_rand_codes((N, K), fmt, 80 + z) for z in range(Z)])
+    ad = torch.stack([_to_dev_codes(a[z], fa) for z in range(Z)])
+    bd = torch.stack([_to_dev_codes(b[z], fmt) for z in range(Z)])
+    g = torch.Generator().manual_seed(91)
+    sx, sw = torch.rand(M, generator=g) + 0.5, torch.rand(N, generator=g) + 0.5
+    bias = torch.randn(N, generator=g)
+    scale = 3000.0 if fmt != O.FMT_E4M3 else 50000.0
+    add = (torch.randn(Z, M, N, generator=g) * scale).to(TDT[dt])
+    kb = K // 2 if fmt == O.FMT_INT4 else K
+    rg = [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
+    want = np.stack([O.gemm_acc(a[z], b[z], fa, fmt) / (sx.numpy().astype(np.float64)[:, None] * sw.numpy().astype(np.float64)[None, :])
+                     + bias.numpy().astype(np.float64) + add[z].float().numpy().astype(np.float64) for z in range(Z)])
+    tol = (4e-6 if dt == "fp32" else 2.0 ** -8) + (3e-4 if fmt == O.FMT_E4M3 else 0.0)
+    tiles = [0, 1, 3, 14] + ([10, 11, 16] if fmt != O.FMT_INT4 else [])
+    for tile in tiles:
+        kw = dict(m=M, n=N, a_fmt=fa, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=kb, bias=bias.to(DEV), tile=tile)
+        if tile == 10:  # the 32 x 32 kernel serves one problem per launch
+            out = torch.stack([ops.gemm(ad[z], bd[z], rg, addend=add[z].contiguous().to(DEV), **kw) for z in range(Z)])
+        else:
+            out = ops.gemm(ad, bd, rg, batch=Z, batch_stride_a=M * K, batch_stride_b=N * kb, addend=add.to(DEV), **kw)
+        assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max(), tile
+    if fmt != O.FMT_INT4:
+        ws = torch.empty(ops.split_bytes(M, N, 4), dtype=torch.uint8, device=DEV)
+        out = ops.gemm(ad[0], bd[0], rg, m=M, n=N, a_fmt=fa, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=kb, bias=bias.to(DEV),
+                       addend=add[0].contiguous().to(DEV), split_k=2, workspace=ws)
+        assert np.abs(_np(out).astype(np.float64) - want[0]).max() <= tol * np.abs(want[0]).max()
+    with pytest.raises(RuntimeError):
+        ops.gemm(ad[0], bd[0], [ops.Range(0, K, None, None)], m=M, n=N, a_fmt=fa, b_fmt=fmt, out_dtype="acc", lda=K, ldb=kb,
+                 addend=add[0].contiguous().to(DEV))
+
+
 @pytest.mark.parametrize("fmt_w", [O.FMT_INT4, O.FMT_INT8])
 @pytest.mark.parametrize("dt", ["fp32", "bf16"])
 def test_group_wise_weight_scales(ops, fmt_w, dt):

@@ -260,6 +260,25 @@ def test_layer_with_the_activation_function_fused_into_its_quantise_kernel(op, g
     assert torch.equal(fake(pre32, pre_op=op, gate=gate32), fake(SegmentLinear._activated(pre32, op, gate32)))
 
 
+def test_layer_hooks_for_smooth_division_and_low_rank_addend():
+    """forward(x, col_div=s, addend=r) == forward(x / s) + r through the fused kernels (the
+    division is exact, the addend joins before the one rounding), and the same on the fake path."""
+    from segquant_amd import workloads as W
+    spec = [s for s in W.config_linears(3, M=160) if s.name == "mlp_up"][0]
+    g = torch.Generator().manual_seed(17)
+    x = (torch.randn(160, spec.K, generator=g)).to(torch.bfloat16).to(DEV)
+    sdiv = (torch.rand(spec.K, generator=g) * 2 + 0.25).to(DEV)
+    add = (torch.randn(160, spec.N, generator=g) * 0.5).to(torch.bfloat16).to(DEV)
+    xs = x / sdiv.to(torch.bfloat16)
+    layer, _ = W.build_layer(spec, device=DEV, real_quant=True, x=xs.float().cpu())
+    want = layer(xs).float() + add.float()
+    got = layer(x, col_div=sdiv, addend=add).float()
+    assert (got - want).abs().max().item() <= 2.0 ** -7 * want.abs().max().item()
+    fake, _ = W.build_layer(spec, device=DEV, real_quant=False, x=xs.float().cpu())
+    x32 = x.float()
+    assert torch.allclose(fake(x32, col_div=sdiv, addend=add.float()), fake(x32 / sdiv) + add.float())
+
+
 def test_reference_named_operators_trace_and_compile():
     """The chunked route calls the reference-named operator through torch.library: opcheck's
     schema / fake-tensor / dispatch checks pass, and a compiled function that calls it gives

@@ -369,3 +369,13 @@ def test_activation_matches_torch_cpu_operators(op, dt):
     # closed-form anchors: gelu(0) = silu(0) = 0, large |x| -> x or 0, odd/even structure
     z = O.activation(np.array([0.0, 30.0, -30.0], dtype=np.float32), op)
     assert z[0] == 0.0 and z[1] == 30.0 and abs(z[2]) < 1e-6
+
+
+@pytest.mark.parametrize("dt", ["fp32", "bf16", "fp16"])
+def test_smooth_divide_is_torchs_in_place_division(dt):
+    tdt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dt]
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(40, 96, generator=g) * 4).to(tdt)
+    s = torch.rand(96, generator=g) * 3 + 0.01
+    want = x.clone().div_(s.to(tdt)).float().numpy()
+    assert np.array_equal(O.smooth_divide(x.float().numpy(), s.numpy(), dt), want)
