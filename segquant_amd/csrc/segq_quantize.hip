@@ -110,9 +110,19 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return ((uint32_t)r & ~nan) | (0x7F7F7F7Fu & nan);
 }
 
+// Four int8 codes in one dword.  Adding 1.5 * 2^23 to the clamped value rounds it to
+// an integer (ties to even, as rintf) and leaves that integer, in two's complement,
+// in the low mantissa bits: the low byte of the sum's bit pattern is the code.  One
+// add instead of round + convert + mask, and three byte permutes per dword.
 __device__ __forceinline__ uint32_t pack4_i8(float a, float b, float c, float d) {
-    return (uint32_t)(q_i8(a) & 0xff) | ((uint32_t)(q_i8(b) & 0xff) << 8) |
-           ((uint32_t)(q_i8(c) & 0xff) << 16) | ((uint32_t)(q_i8(d) & 0xff) << 24);
+    const float magic = 12582912.0f;
+    const uint32_t ua = __float_as_uint(fminf(fmaxf(a, -128.0f), 127.0f) + magic);
+    const uint32_t ub = __float_as_uint(fminf(fmaxf(b, -128.0f), 127.0f) + magic);
+    const uint32_t uc = __float_as_uint(fminf(fmaxf(c, -128.0f), 127.0f) + magic);
+    const uint32_t ud = __float_as_uint(fminf(fmaxf(d, -128.0f), 127.0f) + magic);
+    const uint32_t lo = __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u);  // ua.b0 | ub.b0 << 8
+    const uint32_t hi = __builtin_amdgcn_perm(ud, uc, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);             // lo.b0 lo.b1 hi.b0 hi.b1
 }
 
 // 8 values -> 8 nibbles, element 0 in the lowest nibble.
@@ -425,14 +435,23 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
             const int c = c0 + lane + i * 64;
             if (c < c1) load_run<DT, PRE>(p, xrow, row, c, raw[i]);
         }
+        // short rows: unpack once and keep the floats (64 registers) instead of unpacking
+        // again for the encode; longer rows stay packed
+        constexpr bool KEEP = CPL <= 4;
+        float vf[KEEP ? CPL : 1][16];
         float amax_p = 0.0f, amax_n = 0.0f;
 #pragma unroll
         for (int i = 0; i < CPL; ++i) {
             const int c = c0 + lane + i * 64;
             if (c < c1) {
-                float v[16];
-                raw_to_f32<DT>(raw[i], v);
-                track_amax<DUAL>(v, amax_p, amax_n);
+                if constexpr (KEEP) {
+                    raw_to_f32<DT>(raw[i], vf[i]);
+                    track_amax<DUAL>(vf[i], amax_p, amax_n);
+                } else {
+                    float v[16];
+                    raw_to_f32<DT>(raw[i], v);
+                    track_amax<DUAL>(v, amax_p, amax_n);
+                }
             }
         }
         amax_p = wave_max(amax_p);
@@ -453,9 +472,13 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
         for (int i = 0; i < CPL; ++i) {
             const int c = c0 + lane + i * 64;
             if (c < c1) {
-                float v[16];
-                raw_to_f32<DT>(raw[i], v);
-                encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
+                if constexpr (KEEP) {
+                    encode16<FMT>(p, row, (int64_t)c << 4, vf[i], s_pos, s_neg, two);
+                } else {
+                    float v[16];
+                    raw_to_f32<DT>(raw[i], v);
+                    encode16<FMT>(p, row, (int64_t)c << 4, v, s_pos, s_neg, two);
+                }
             }
         }
     }
