@@ -134,3 +134,60 @@ def test_full_size_dynamic_quantize_against_oracle(ops, K, fmt):
     assert np.array_equal(scale.cpu().numpy(), want_s)
     want = O.quantize_act(xn[None], want_s, fmt)[0]
     assert np.array_equal(codes.cpu().numpy().view(np.uint8), want.view(np.uint8))
+
+
+@pytest.mark.parametrize("M,K,N", [(8192, 1280, 10240), (8192, 5120, 1280), (2048, 1280, 10240)])
+def test_full_size_group_wise_scales_product_check(ops, M, K, N):
+    """Configuration 4 at full size with one weight scale per 128 input channels, int4 weights
+    expanded into the lent workspace: out r == sum_g A_g (W_g^T (r / sw_g)) / sx."""
+    G = 128
+    a, b = _codes((M, K), O.FMT_INT8, 120), _codes((N, K), O.FMT_INT4, 121)
+    g = np.random.default_rng(122)
+    sx = (g.random(M) + 0.5).astype(np.float32)
+    swg = (g.random((K // G, N)) + 0.5).astype(np.float32)  # (groups, N)
+    factors = torch.from_numpy((1.0 / swg.astype(np.float64)).astype(np.float32)).to(DEV)
+    one = torch.ones(1, device=DEV)
+    out = ops.gemm(_dev(a, O.FMT_INT8), _dev(b, O.FMT_INT4), [ops.Range(0, K, torch.from_numpy(sx).to(DEV), one, 0, 1, 0)],
+                   m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT4, out_dtype=torch.float32, lda=K, ldb=K // 2,
+                   workspace=ops.int4_workspace(DEV, N * K), group_dequant=factors)
+    f = factors.double().cpu().numpy()
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    r = g.integers(-1, 2, size=N).astype(np.float64)
+    l = g.integers(-1, 2, size=M).astype(np.float64)
+    right = np.zeros(M)
+    left = np.zeros(N)
+    la = l / sx.astype(np.float64)
+    for j in range(K // G):
+        sl = slice(j * G, (j + 1) * G)
+        right += a64[:, sl] @ (b64[:, sl].T @ (r * f[j]))
+        left += ((la @ a64[:, sl]) @ b64[:, sl].T) * f[j]
+    right /= sx.astype(np.float64)
+    # fp32 accumulation over K / 128 groups, then a sum of up to 10240 signed entries: an error of a
+    # few 1e-7 per entry, measured against the entries' size
+    c = out.double().cpu().numpy()
+    assert np.abs(c @ r - right).max() <= 2e-6 * max(np.abs(right).max(), np.sqrt(N) * np.abs(c).max())
+    assert np.abs(l @ c - left).max() <= 2e-6 * max(np.abs(left).max(), np.sqrt(M) * np.abs(c).max())
+
+
+@pytest.mark.parametrize("M", [1024, 4608])
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+def test_full_size_config5_ranges_parked_or_split(ops, M, fmt):
+    """Configuration 5 (K = 3072 | 12288, the second segment read from two code tensors) with the
+    workspace the layer lends: int8 parks its finished ranges, 1024 tokens of e4m3 share the K
+    steps of a tile between workgroups.  Same answer as the launch without a workspace (second
+    accumulator set / in-place rescaling, one workgroup per tile), to fp32 summation order."""
+    K0, K1, N = 3072, 12288, 3072
+    K = K0 + K1
+    a, a2, b = _codes((M, K), fmt, 130), _codes((M, K), fmt, 131), _codes((N, K), fmt, 132)
+    ad, a2d, bd = _dev(a, fmt), _dev(a2, fmt), _dev(b, fmt)
+    g = torch.Generator().manual_seed(133)
+    s0 = (torch.rand(1, generator=g) + 0.5).to(DEV)
+    sx, sx2 = (torch.rand(M, generator=g) + 0.5).to(DEV), (torch.rand(M, generator=g) + 0.5).to(DEV)
+    sw, bias = (torch.rand(N, generator=g) + 0.5).to(DEV), torch.randn(N, generator=g).to(DEV)
+    rg = [ops.Range(0, K0, s0, sw, 0, 0, 1), ops.Range(K0, K1, sx, sw, 0, 1, 1), ops.Range(K0, K1, sx2, sw, 1, 1, 1)]
+    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, bias=bias, a_neg=a2d)
+    plain = ops.gemm(ad, bd, rg, split_k=1, **kw)
+    nbytes = max(ops.park_bytes(M, N), ops.split_bytes(M, N, max(ops.auto_splits(M, N, (K0 + 2 * K1) // 128), 1)))
+    lent = ops.gemm(ad, bd, rg, workspace=torch.empty(nbytes, dtype=torch.uint8, device=DEV), **kw)
+    tol = 3e-6 if fmt == O.FMT_INT8 else 2e-4
+    assert (lent - plain).abs().max().item() <= tol * plain.abs().max().item()
