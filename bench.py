@@ -33,9 +33,10 @@ GEMM_KERNELS = {
 MEASURED_TRAFFIC_BYTES = {3: 343.5e6}
 
 
-def cpu_baseline(specs, rows, repeats=3):
+def cpu_baseline(specs, rows, repeats=5):
     """The fake-quant path (fp32 quantise->de-quantise + torch matmul) on the
-    host cores, on the first ``rows`` tokens of every linear of the workload."""
+    host cores, on the first ``rows`` tokens of every linear of the workload
+    (0: all of them)."""
     import torch
     from oracle import fake_path_torch as F
     from segquant_amd import workloads as W
@@ -45,10 +46,14 @@ def cpu_baseline(specs, rows, repeats=3):
     work = []
     ops = 0
     for sp in specs:
-        x = W.make_input(sp, M=rows)
+        rows_sp = min(rows, sp.M) if rows > 0 else sp.M
+        x = W.make_input(sp, M=rows_sp)
         w = W.make_weight(sp)
         # weights are fake-quantised once, offline, and stored de-quantised
-        if sp.weight_axis == 1:
+        if sp.weight_axis == 1 and sp.weight_group:
+            wg = w.reshape(w.shape[0], -1, sp.weight_group)
+            w_hat = F.fake_quant(wg, sp.weight, F.scale_of(wg.abs().amax(dim=2, keepdim=True), sp.weight)).reshape(w.shape)
+        elif sp.weight_axis == 1:
             ws = F.scale_of(w.abs().amax(dim=1, keepdim=True), sp.weight)
             w_hat = F.fake_quant(w, sp.weight, ws)
         elif sp.seg_mode == "weight" and sp.chunksizes:
@@ -60,7 +65,7 @@ def cpu_baseline(specs, rows, repeats=3):
         n_in = len(bounds) - 1
         dual = [i in sp.dual_segments for i in range(n_in)]
         work.append((x, w_hat, W.make_bias(sp), sp.act, bounds, dual, sp.act_axis == -1))
-        ops += 2 * rows * sp.N * sp.K
+        ops += 2 * rows_sp * sp.N * sp.K
     times = []
     for it in range(repeats + 1):
         t0 = time.perf_counter()
@@ -71,7 +76,8 @@ def cpu_baseline(specs, rows, repeats=3):
             times.append(t1 - t0)
     t = sorted(times)[len(times) // 2]
     return {"value": ops / t / 1e12, "unit": "TOP/s", "cores": threads, "kind": "port",
-            "sample": f"first {rows} of {specs[0].M} tokens of each linear, fp32 fake-quant + torch.matmul, "
+            "sample": (f"first {rows} tokens" if rows > 0 else "all tokens") +
+                      f" of each linear of the workload ({specs[0].M} for the first), fp32 fake-quant + torch.matmul, "
                       f"median of {repeats} passes, {t:.3f} s per pass"}
 
 
@@ -84,7 +90,8 @@ def main():
                     help="untimed steps before the warm-up: the first ~25 steps after start-up run ~10 %% slower "
                          "(measured: 606 us against 547 us per step) while clocks and page tables settle")
     ap.add_argument("--config", type=int, default=3, help="benchmark configuration 1..5 (default: FLUX int8, M=4608)")
-    ap.add_argument("--cpu-rows", type=int, default=512, help="tokens per linear in the CPU baseline sample")
+    ap.add_argument("--cpu-rows", type=int, default=0,
+                    help="tokens per linear in the CPU baseline sample (0: the whole workload; a few seconds for config 3)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")

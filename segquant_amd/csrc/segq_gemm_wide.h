@@ -109,34 +109,40 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
                 for (int v = 0; v < 4; ++v) bvv[a][v] = p.bias ? load_bias(p.bias, p.bias_dtype, n_base + a * 16 + v) : 0.0f;
             }
         }
+        // (two instances, so that launches without an addend carry no trace of it)
+        auto blocks = [&](auto add_c) __attribute__((always_inline)) {
+            constexpr bool ADD = decltype(add_c)::value;
 #pragma unroll
-        for (int b = 0; b < TM; ++b) {
+            for (int b = 0; b < TM; ++b) {
 #pragma unroll
-            for (int a = 0; a < TN; ++a) {
-                float o[4];
+                for (int a = 0; a < TN; ++a) {
+                    float o[4];
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    o[v] = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
-                add_addend4(p, z, min(m_base + b * 16, p.M - 1), n_base + a * 16, o);
-                const bool bf = p.out_dtype == SEGQ_BF16;
-                *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
-                    make_uint2(bf ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]),
-                               bf ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]));
-            }
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int j = 0; j < (16 * CH + 63) / 64; ++j) {
-                const int c = j * 64 + lane;
-                const int row = c / CH, col = c % CH;
-                if ((16 * CH) % 64 != 0 && c >= 16 * CH) continue;
-                const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + col * 16);
-                const int m = m0 + wm * WM + b * 16 + row;
-                if (m < p.M) {
-                    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + col * 8) = v;
+                    for (int v = 0; v < 4; ++v)
+                        o[v] = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
+                    if constexpr (ADD) add_addend4(p, z, min(m_base + b * 16, p.M - 1), n_base + a * 16, o);
+                    const bool bf = p.out_dtype == SEGQ_BF16;
+                    *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
+                        make_uint2(bf ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]),
+                                   bf ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]));
                 }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int j = 0; j < (16 * CH + 63) / 64; ++j) {
+                    const int c = j * 64 + lane;
+                    const int row = c / CH, col = c % CH;
+                    if ((16 * CH) % 64 != 0 && c >= 16 * CH) continue;
+                    const uint4 v = *reinterpret_cast<const uint4*>(patch + row * RS + col * 16);
+                    const int m = m0 + wm * WM + b * 16 + row;
+                    if (m < p.M) {
+                        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.C) + c_off + (int64_t)m * p.ldc + n0 + wn * WN + col * 8) = v;
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_wave_barrier();
-        }
+        };
+        if (p.addend) blocks(std::true_type{});
+        else blocks(std::false_type{});
         return;
     }
 #pragma unroll
