@@ -93,6 +93,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=0,
                     help="tokens per linear in the CPU baseline sample (0: the whole workload; a few seconds for config 3)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-e4m3", action="store_true", help="skip the supplementary e4m3 pass over the config-3 shapes")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")
     args = ap.parse_args()
@@ -189,6 +190,30 @@ def main():
                      "unit": "GB/s", "frac": round(q_gbs / PEAK_HBM, 4), "launches": n_q,
                      "avg_launch_us": round(q_t / max(n_q, 1) * 1e6, 2)},
     }
+    if args.config == 3 and not args.no_e4m3:
+        # Supplementary: the same three shapes with e4m3 codes on both sides (the metric names
+        # int8 and fp8 peaks alike), GEMM launches only, same rotation of operands.
+        import dataclasses
+        del sets, layers
+        torch.cuda.empty_cache()
+        specs8 = [dataclasses.replace(sp, act="fpe4m3", weight="fpe4m3") for sp in specs]
+        layers8 = [W.build_layer(sp, device=dev, real_quant=True)[0] for sp in specs8]
+        sets8 = [[x.to(dev).clone() for x in inputs] for _ in range(n_sets)]
+        for i in range(20):
+            for layer, x in zip(layers8, sets8[i % n_sets]):
+                layer(x)
+        with ops.record_launches() as log8:
+            for i in range(20):
+                for layer, x in zip(layers8, sets8[i % n_sets]):
+                    layer(x)
+            torch.cuda.synchronize()
+        t8 = sum(e0.elapsed_time(e1) for kind, e0, e1, _ in log8 if kind == "gemm") * 1e-3
+        n8 = sum(1 for kind, *_ in log8 if kind == "gemm")
+        ops8 = sum(2.0 * info["m"] * info["n"] * info["k_alg"] for kind, _, _, info in log8 if kind == "gemm")
+        out["e4m3_same_shapes"] = {"bound": "mfma", "kernel": "segq::gemm_pipe_kernel<192,288> / <288,192> (e4m3)",
+                                   "achieved": round(ops8 / t8 / 1e12, 2), "peak": PEAK_TOPS["fpe4m3"], "unit": "TFLOP/s",
+                                   "frac": round(ops8 / t8 / 1e12 / PEAK_TOPS["fpe4m3"], 4), "launches": n8,
+                                   "avg_launch_us": round(t8 / max(n8, 1) * 1e6, 2)}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(specs, args.cpu_rows)
     print(json.dumps(out))
