@@ -263,8 +263,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         return d->workspace_bytes >= tiles * t.bm * t.bn * 4;
     };
     if (d->tile == 0) {
-        if (groups) cfg = FIRST_WIDE_CFG + 3;  // the one tile the group kernel is built for
-        else {
+        if (groups) {
+            // 128 x 128: at 126 registers two workgroups share a CU, and one's conversion (VALU) runs under
+            // the other's MFMAs; measured 8 % (8192 x 10240 x 1280) to 25 % (8192 x 1280 x 5120) ahead
+            // of 256 x 128 / 128 x 256, which are selectable by id
+            cfg = FIRST_WIDE_CFG + 3;
+        } else {
             cfg = park ? choose_tile(d->m, d->n, d->batch, false, wide_ok, plain8) : -1;
             park = park && park_fits(cfg);
             if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
@@ -330,10 +334,11 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     } else if (cfg >= FIRST_WIDE_CFG) {
         if (!wide_ok) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs K ranges in multiples of 128", cfg + 1);
         if (fold2 && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
-        if (groups && cfg != FIRST_WIDE_CFG + 3)
-            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tile %d only", FIRST_WIDE_CFG + 4);
+        if (groups && cfg == FIRST_WIDE_CFG) cfg = FIRST_WIDE_CFG + 1;
+        if (groups && cfg > FIRST_WIDE_CFG + 3)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tiles %d to %d", FIRST_WIDE_CFG + 2, FIRST_WIDE_CFG + 4);
     } else if (groups) {
-        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tile %d only", FIRST_WIDE_CFG + 4);
+        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on tiles %d to %d", FIRST_WIDE_CFG + 2, FIRST_WIDE_CFG + 4);
     } else if (cfg >= FIRST_BIG_CFG) {
         if (!wide_ok || w4 || fold)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs one range, 8-bit weights and K in multiples of 128", cfg + 1);

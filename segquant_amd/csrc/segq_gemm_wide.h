@@ -462,11 +462,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // sums are multiplied by the factors and added to an fp32 set, which from
     // there on is treated like e4m3's fp32 accumulators: in units of the current
     // range, rescaled at range boundaries, scaled by 1/(sx sw) in the epilogue.
-    // The conversion of step s runs between the MFMAs of step s + 1's first
-    // half, each accumulator right before the MFMA that restarts it from zero
-    // (two int32 sets taking turns, so that the conversion spreads over the whole
-    // step, measured no faster: the kernel is held by its one workgroup per CU).
+    // The group kernel runs the e4m3 schedule (whole-step fragments of 32 bytes,
+    // refilled as the step lets go of them): both 64-byte K halves of an output
+    // block are multiplied back to back into a handful of int32 temporaries,
+    // which are converted at once, so no int32 accumulator set lives across
+    // steps and the 64 x 64 wave tile fits.
     static_assert(!GRP || (!F8 && NS == 2), "group factors: int8, two stages");
+    constexpr bool S8 = F8 || GRP;  // whole-step fragments
     //
     // PARK (int8, several ranges): no second register set at all.  When a range
     // ends, its int32 sums are converted to the LAST range's units
@@ -487,7 +489,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     int r_last = p.nr - 1, r_begin = 0;  // (r_begin: the range its first step lies in)
 
     static_assert(NS >= 2 && (NS - 1) * (A_IT + B_IT) < 64, "vmcnt holds 6 bits");
-    static_assert(!F8 || (NS == 2 && TN >= 3), "the e4m3 schedule reads two weight fragments ahead in a two-stage ring");
+    static_assert(!S8 || (NS == 2 && TN >= 3), "the e4m3 schedule reads two weight fragments ahead in a two-stage ring");
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t* const As = smem;                  // [NS][BM][128]
     uint8_t* const Bs = smem + NS * BM * BK;   // [NS][BN][128]
@@ -578,10 +580,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // int8: two fragment sets, one per 64-byte K half of a step.  e4m3: one set of
     // 32-byte fragments (the 16 x 16 x 128 MFMA eats a whole step), whose registers
     // are refilled for the next step as the current one lets go of them.
-    v4i fa[F8 ? 1 : 2][F8 ? 1 : TM], fb[F8 ? 1 : 2][F8 ? 1 : TN];
-    v8i fa8[F8 ? TM : 1], fb8[F8 ? TN : 1];
+    v4i fa[S8 ? 1 : 2][S8 ? 1 : TM], fb[S8 ? 1 : 2][S8 ? 1 : TN];
+    v8i fa8[S8 ? TM : 1], fb8[S8 ? TN : 1];
     auto frag8 = [&](int buf, int i) {  // fragment i of the step in buffer buf: 0 .. TM-1 activations, then weights
-      if constexpr (F8) {
+      if constexpr (S8) {
         const int off0 = ((2 * lgrp) ^ f_sw) << 4;
         const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
         const uint8_t* src = (i < TM) ? As + buf * BM * BK + a_frag + i * 16 * BK : Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK;
@@ -596,7 +598,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // K half h of the tile in buffer buf -> fragment slot h, one 16-byte read at a
     // time: reads 0 .. TM-1 are the activation fragments, TM .. TM+TN-1 the weights
     auto frag1 = [&](int buf, int h, int i) {
-        if constexpr (!F8) {
+        if constexpr (!S8) {
             const int off = ((h * 4 + lgrp) ^ f_sw) << 4;
             if (i < TM) fa[h][i] = *reinterpret_cast<const v4i*>(As + buf * BM * BK + a_frag + i * 16 * BK + off);
             else fb[h][i - TM] = *reinterpret_cast<const v4i*>(Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK + off);
@@ -608,20 +610,6 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     };
     const int m_base = m0 + wm * WM + lrow;
     const int n_base = n0 + wn * WN + 4 * lgrp;
-    // the group factors of the step in ring slot `slot` times this step's sums, into the fp32 set
-    auto add_groups = [&](auto& set, const float* grw, int slot) __attribute__((always_inline)) {
-        if constexpr (GRP) {
-#pragma unroll
-            for (int a = 0; a < TN; ++a) {
-                const v4f g = *reinterpret_cast<const v4f*>(grw + slot * BN + wn * WN + a * 16 + 4 * lgrp);
-#pragma unroll
-                for (int b = 0; b < TM; ++b) {
-                    accf[a][b] += __builtin_convertvector(set[a][b], v4f) * g;
-                    set[a][b] = acc_zero;
-                }
-            }
-        }
-    };
     v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (BM * BN / 4) + tid : nullptr;
     auto park = [&](int r) __attribute__((always_inline)) {
         if constexpr (PARK) {
@@ -751,10 +739,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     constexpr int EPI_FLOATS = BM + 2 * BN, EPI_IT = (EPI_FLOATS + NT - 1) / NT;
     float* const epi = reinterpret_cast<float*>(smem + NS * (BM + BN) * BK);
     // group factors: a ring of four rows of BN floats behind the epilogue's vectors.  The row of
-    // step s arrives with the step's operands and is read all through step s + 1, at whose end
-    // the row of step s + 3 is already on its way: it must not land in the same slot
+    // step s arrives with the step's operands and is read all through step s, at whose end the
+    // row of step s + 2 is already on its way
     float* const grw = epi + EPI_FLOATS;
-    int lslot = 0, cslot = 0, pslot = 0;  // slots of the step being loaded / multiplied / converted
+    int lslot = 0, cslot = 0;  // slots of the step being loaded / multiplied
     auto dma_g = [&]() {
         if constexpr (GRP) {
             if (wave < BN / 64) {
@@ -802,7 +790,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         if (e < EPI_FLOATS) epi[e] = (e < BM + BN && !ACCF) ? __builtin_amdgcn_rcpf(epi_val[i]) : epi_val[i];
     }
     __syncthreads();
-    if constexpr (F8) {
+    if constexpr (S8) {
 #pragma unroll
         for (int i = 0; i <= TM; ++i) frag8(0, i);  // activations and the first weight fragment
     } else {
@@ -830,19 +818,44 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // registers this step is done with: next weight fragment 0, then each
     // activation fragment right behind the last MFMA that reads it, with the DMA
     // of step s + 2 spread over the same MFMAs.
-    auto step8 = [&](auto dma_c, auto more_c) {
+    auto step8 = [&](auto dma_c, auto more_c) __attribute__((always_inline)) {
         constexpr bool DMA_ = decltype(dma_c)::value;
         constexpr bool MORE_ = decltype(more_c)::value;
         constexpr int NDM8 = A_IT + B_IT, TAIL = 2 * TM;  // DMA instructions over the tail's MFMAs
         const int nbuf = buf ^ 1;
+        // group mode: an output block is both K halves of the step into an int32 temporary
+        // (first MFMA with a zero C operand), converted and scaled by this step's factors at once
+        auto lo4 = [](const v8i& f) __attribute__((always_inline)) { return v4i{f[0], f[1], f[2], f[3]}; };
+        auto hi4 = [](const v8i& f) __attribute__((always_inline)) { return v4i{f[4], f[5], f[6], f[7]}; };
+        const float* const gsrc = grw + cslot * BN + wn * WN + 4 * lgrp;
 #pragma unroll
         for (int a = 0; a < TN - 2; ++a) {
+            if constexpr (GRP) {
+                v4i t[TM];
+                const v4f g = *reinterpret_cast<const v4f*>(gsrc + a * 16);
 #pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                if (b == 0 && a == 0) frag8(buf, TM + 1);
-                if (b == (TM > 1 ? 1 : 0)) frag8(buf, TM + a + 2);
-                acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int b = 0; b < TM; ++b) {
+                    if (b == 0 && a == 0) frag8(buf, TM + 1);
+                    if (b == (TM > 1 ? 1 : 0)) frag8(buf, TM + a + 2);
+                    t[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo4(fb8[a]), lo4(fa8[b]), acc_zero, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    t[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi4(fb8[a]), hi4(fa8[b]), t[b], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int b = 0; b < TM; ++b) accf[a][b] += __builtin_convertvector(t[b], v4f) * g;
+            } else {
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if (b == 0 && a == 0) frag8(buf, TM + 1);
+                    if (b == (TM > 1 ? 1 : 0)) frag8(buf, TM + a + 2);
+                    if constexpr (F8)
+                        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         wait_dma(std::integral_constant<int, 0>{});
@@ -851,19 +864,47 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         const uint8_t* const bp = Bb + lk;
 #pragma unroll
         for (int a = TN - 2; a < TN; ++a) {
+            if constexpr (GRP) {
+                v4i t[TM];
+                const v4f g = *reinterpret_cast<const v4f*>(gsrc + a * 16);
 #pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
-                const int j = (a - (TN - 2)) * TM + b;
-                if constexpr (DMA_) {
+                for (int b = 0; b < TM; ++b) {
+                    t[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo4(fb8[a]), lo4(fa8[b]), acc_zero, 0, 0, 0);
+                    const int j = (a - (TN - 2)) * TM + b;
+                    if constexpr (DMA_) {
 #pragma unroll
-                    for (int i = j * NDM8 / TAIL; i < (j + 1) * NDM8 / TAIL; ++i) dma1(ap, bp, buf, i);
+                        for (int i = j * NDM8 / TAIL; i < (j + 1) * NDM8 / TAIL; ++i) dma1(ap, bp, buf, i);
+                        if (j == TAIL - 1) dma_g();
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr (MORE_) {
-                    if (a == TN - 2 && b == 0) frag8(nbuf, TM);  // next weight fragment 0: its registers were free since block 0
-                    if (a == TN - 1) frag8(nbuf, b);              // next activation fragment b: this was its last reader
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    t[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi4(fb8[a]), hi4(fa8[b]), t[b], 0, 0, 0);
+                    if constexpr (MORE_) {
+                        if (a == TN - 2 && b == 0) frag8(nbuf, TM);  // next weight fragment 0: free since block 0
+                        if (a == TN - 1) frag8(nbuf, b);              // next activation fragment b: this was its last reader
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < TM; ++b) accf[a][b] += __builtin_convertvector(t[b], v4f) * g;
+            } else {
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if constexpr (F8)
+                        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb8[a], fa8[b], acc[a][b], 0, 0, 0, 0, 0, 0);
+                    const int j = (a - (TN - 2)) * TM + b;
+                    if constexpr (DMA_) {
+#pragma unroll
+                        for (int i = j * NDM8 / TAIL; i < (j + 1) * NDM8 / TAIL; ++i) dma1(ap, bp, buf, i);
+                    }
+                    if constexpr (MORE_) {
+                        if (a == TN - 2 && b == 0) frag8(nbuf, TM);  // next weight fragment 0: its registers were free since block 0
+                        if (a == TN - 1) frag8(nbuf, b);              // next activation fragment b: this was its last reader
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         // A full LDS wait: the last activation fragments were read a few MFMAs ago
@@ -873,6 +914,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         __builtin_amdgcn_s_waitcnt(0xC07F);
         if constexpr (DMA_) advance_load();
         ck += BK;
+        cslot = (cslot + 1) & 3;
         if (ck >= ck1) {
             if constexpr (FOLD) fold(cr);
             ++cr;
@@ -886,29 +928,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         constexpr bool DMA_ = decltype(dma_c)::value;
         constexpr bool MORE_ = decltype(more_c)::value;
         const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
-        // group schedule: the previous step's factors, one column block ahead of their use
-        // (the first step adds zeros)
-        const float* const gsrc = grw + pslot * BN + wn * WN + 4 * lgrp;
-        v4f gv = {0.f, 0.f, 0.f, 0.f}, gnext = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (GRP) gnext = *reinterpret_cast<const v4f*>(gsrc);
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
                 const int i = a * TM + b;
-                if constexpr (GRP) {
-                    if (b == 0) {
-                        gv = gnext;
-                        if (a + 1 < TN) gnext = *reinterpret_cast<const v4f*>(gsrc + (a + 1) * 16);
-                    }
-                }
                 if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(buf, 1, i / RD_EVERY);
-                if constexpr (GRP) {
-                    accf[a][b] += __builtin_convertvector(acc[a][b], v4f) * gv;
-                    acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc_zero, 0, 0, 0);
-                } else {
-                    acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
-                }
+                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
@@ -926,7 +952,6 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 const int i = a * TM + b;
                 if constexpr (DMA_) {
                     if (i % DM_EVERY == DM_EVERY - 1 && i / DM_EVERY < NDM) dma1(ap, bp, buf, i / DM_EVERY);
-                    if (i == NMF - 1) dma_g();
                 }
                 if constexpr (MORE_) {
                     if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(nbuf, 0, i / RD_EVERY);
@@ -941,11 +966,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0), vmcnt untouched
         if constexpr (DMA_) advance_load();
         ck += BK;
-        pslot = cslot;
-        cslot = (cslot + 1) & 3;
         dirty = true;
         if (ck >= ck1) {  // the range is complete: fold it, move to the next one
-            if constexpr (GRP && FOLD) add_groups(acc, grw, pslot);  // this step's sums are still in the old range's units
             if constexpr (PARK) park(cr);
             else if constexpr (FOLD) fold(cr);
             dirty = false;
@@ -957,7 +979,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         buf = nbuf;
     };
     auto step = [&](auto dma_c, auto more_c) __attribute__((always_inline)) {
-        if constexpr (F8) step8(dma_c, more_c);
+        if constexpr (S8) step8(dma_c, more_c);
         else step_i8(dma_c, more_c);
     };
     int s = 0;
@@ -968,7 +990,6 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         if (dirty) fold(cr);
     }
     if constexpr (GRP) {
-        add_groups(acc, grw, pslot);  // the last step's sums
         v4f none[1][1];
         wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, false>(p, accf, none, smem, z, m0, n0, wave, lane, r_epi, epi);
     } else if constexpr (PARK) {
@@ -1032,12 +1053,18 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
     if constexpr (!B4 && FMT == GEMM_I8) {
         if (p.grw) {  // group-wise factors (the host has checked: plain codes, K ranges in whole steps)
             if (asel) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need plain codes");
-            // one tile only: with a second accumulator set, the factors and the conversion's
-            // temporaries the 64 x 64 wave tiles of 256 x 128 and 128 x 256 spill ~100 registers
-            if (wcfg == 3)
-                return fold ? launch_pipe_instance<128, 128, 2, 4, FMT, true, 2, true>(p, batch, st)
-                            : launch_pipe_instance<128, 128, 2, 4, FMT, false, 2, true>(p, batch, st);
-            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on the 128x128 tile of eight waves");
+            switch (wcfg) {
+                case 0: case 1:
+                    return fold ? launch_pipe_instance<256, 128, 4, 2, FMT, true, 2, true>(p, batch, st)
+                                : launch_pipe_instance<256, 128, 4, 2, FMT, false, 2, true>(p, batch, st);
+                case 2:
+                    return fold ? launch_pipe_instance<128, 256, 2, 4, FMT, true, 2, true>(p, batch, st)
+                                : launch_pipe_instance<128, 256, 2, 4, FMT, false, 2, true>(p, batch, st);
+                case 3:
+                    return fold ? launch_pipe_instance<128, 128, 4, 2, FMT, true, 2, true>(p, batch, st)
+                                : launch_pipe_instance<128, 128, 4, 2, FMT, false, 2, true>(p, batch, st);
+            }
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on the 256x128, 128x256 and 128x128 tiles of eight waves");
         }
     }
     if constexpr (!B4) {

@@ -578,19 +578,22 @@ def test_group_wise_weight_scales(ops, fmt_w, dt):
     kw = dict(m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=fmt_w, out_dtype=TDT[dt], lda=K, ldb=K // 2 if fmt_w == O.FMT_INT4 else K,
               bias=bias.to(DEV), workspace=ws, group_dequant=factors)
     tol = 4e-6 if dt == "fp32" else 2.0 ** -8
-    # (a) one range, per-token scales
-    out = ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 0, 1, 0)], **kw)
+    # (a) one range, per-token scales, on each of the tiles the group kernel is built for
     want = O.linear_groups(a, want_codes, sx.numpy(), sw, G, bias.numpy())
-    assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max()
+    for tile in (0, 12, 13, 14):
+        out = ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 0, 1, 0)], tile=tile, **kw)
+        assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max(), tile
     # (b) K segments [0, 512) and [512, 1280); the second read twice, from two code tensors
     rg = [ops.Range(0, 512, sx.to(DEV), one, 0, 1, 0), ops.Range(512, K - 512, sx2.to(DEV), one, 0, 1, 0),
           ops.Range(512, K - 512, sx.to(DEV), one, 1, 1, 0)]
-    out = ops.gemm(ad, codes, rg, a_neg=a2d, **kw)
+    outs = [ops.gemm(ad, codes, rg, a_neg=a2d, tile=tile, **kw) for tile in (12, 13, 14)]
+    out = outs[2]
     nog = O.linear_groups  # per part: groups are indexed by absolute K, so slice the scales with the codes
     want = (nog(a[:, :512], want_codes[:, :512], sx.numpy(), sw[:, :4], G) +
             nog(a[:, 512:], want_codes[:, 512:], sx2.numpy(), sw[:, 4:], G) +
             nog(a2[:, 512:], want_codes[:, 512:], sx.numpy(), sw[:, 4:], G) + bias.numpy().astype(np.float64))
-    assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max()
+    for o in outs:
+        assert np.abs(_np(o).astype(np.float64) - want).max() <= tol * np.abs(want).max()
     # what the group kernel does not serve is refused, not approximated
     with pytest.raises(RuntimeError):
         ops.gemm(ad, codes, [ops.Range(0, K, sx.to(DEV), one, 2, 1, 0)], **kw)
