@@ -33,12 +33,19 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 // tiles of 256 x 256 beat 432 tiles of 256 x 128 by 30 %).  The 192 x 288 and
 // 288 x 192 tiles exist because 4608 rows of FLUX tokens make whole rounds with
 // them where 256 x 256 leaves the last round half empty.
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8) {  // fold: needs a second accumulator set
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8, int64_t k_steps = 1 << 20) {  // fold: needs a second accumulator set
     auto tiles = [&](int cfg) {
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
     };
     if (wide_ok && tiles(FIRST_WIDE_CFG + 3) >= 96) {
+        // Short contractions of middling size: the plain 128 x 128 kernel needs ~100 registers, so two
+        // workgroups share a CU and each one's prologue and epilogue (most of a tile's time at a dozen
+        // K steps) run under the other's MFMAs.  Measured at K = 1280 .. 1536: 2048 x 10240 34.5 vs 45.5 us
+        // and 4096 x 6144 44.7 vs 47-50 us for the rule below's choice; 8192 x 10240 (1280 tiles of
+        // 256 x 256, five whole rounds) stays 20 % better on the big tile.
+        if (plain8 && !fold && k_steps <= 12 && tiles(FIRST_WIDE_CFG) <= 512 && tiles(FIRST_WIDE_CFG + 3) >= 512)
+            return FIRST_WIDE_CFG + 3;
         static const double weight[6] = {1.0, 1.18, 1.18, 1.45, 1.04, 1.04};
         const int64_t cus = 256;
         int best = -1;
@@ -271,7 +278,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         } else {
             cfg = park ? choose_tile(d->m, d->n, d->batch, false, wide_ok, plain8) : -1;
             park = park && park_fits(cfg);
-            if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8);
+            if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8, ktotal / 128);
         }
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
