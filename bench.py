@@ -25,7 +25,7 @@ PEAK_HBM = 8000.0                               # GB/s
 # the GEMM kernels the tile heuristic picks for each configuration's linears (rocprofv3 traces, profiles/)
 GEMM_KERNELS = {
     1: "segq::gemm_kernel (int8, general)",
-    2: "segq::gemm_pipe_kernel<192,288> / <256,128, two ranges> (e4m3)",
+    2: "segq::gemm_pipe_kernel<128,128> / <256,128, two ranges> (e4m3)",
     3: "segq::gemm_pipe_kernel<192,288> / <288,192> (int8)",
     4: "segq::gemm_pipe_kernel<128,128, group factors> (int8 x int4 expanded to int8)",
     5: "segq::gemm_pipe_kernel<288,192> / <128,128> (int8 with parked ranges, e4m3 rescaled in place)",
