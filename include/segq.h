@@ -249,6 +249,13 @@ int segq_gemm(const segq_gemm_desc* d, segq_stream_t stream);
 /* Number of tile configurations accepted in segq_gemm_desc.tile (ids 1..count). */
 int segq_gemm_tile_count(void);
 
+/* *bytes = the workspace the launch described by d would use if the caller lent as much as the
+ * library can make use of (0: it has no use for one).  d is the descriptor of the launch itself;
+ * its own workspace fields are ignored, nothing is enqueued.  Callers size the buffer they lend
+ * with this instead of restating the library's rules.  Replaces nothing in the reference, which
+ * allocates its temporaries itself (segquant/src/real_quant/real_gemm.cu:684-698, :855-865). */
+int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes);
+
 /* Quantise-then-multiply in one call: q writes its codes into a caller-provided
  * workspace that g reads as its a (and a_neg).  Replaces the body of
  * real_quantized_gemm_scaled / real_quantized_gemm_dual_scaled

@@ -1,6 +1,7 @@
 // C ABI of libsegq: argument checks, kernel selection, launches.
 #include "segq_gemm_kernel.h"
 #include <string.h>
+#include <atomic>
 
 namespace segq {
 
@@ -17,6 +18,30 @@ int fail(int status, const char* fmt, ...) {
 int check_launch(const char* what) {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(SEGQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return SEGQ_OK;
+}
+
+int device_cus() {
+    static std::atomic<int> cus[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+int reserve_lds(const void* kern, int bytes, unsigned long long* done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (__atomic_load_n(done, __ATOMIC_ACQUIRE) & bit) return SEGQ_OK;
+    // (the call is idempotent: two threads that both find the bit clear both make it)
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+        return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", bytes);
+    __atomic_fetch_or(done, bit, __ATOMIC_RELEASE);
     return SEGQ_OK;
 }
 
@@ -47,7 +72,7 @@ static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide
         if (plain8 && !fold && k_steps <= 12 && tiles(FIRST_WIDE_CFG) <= 512 && tiles(FIRST_WIDE_CFG + 3) >= 512)
             return FIRST_WIDE_CFG + 3;
         static const double weight[6] = {1.0, 1.18, 1.18, 1.45, 1.04, 1.04};
-        const int64_t cus = 256;
+        const int64_t cus = device_cus();
         int best = -1;
         double best_cost = 0;
         for (int i = 0; i < 6; ++i) {
@@ -136,7 +161,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* part, i
     }
 }
 
-static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
+// need != nullptr: nothing is launched; *need receives the workspace bytes the launch would use if
+// the caller lent as much as the library can make use of.
+static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, int64_t* need = nullptr) {
+    if (need) *need = 0;
     if (!d) return fail(SEGQ_ERR_ARG, "segq_gemm: null descriptor");
     if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
     if (d->m == 0 || d->n == 0) return SEGQ_OK;
@@ -163,6 +191,8 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
                                               "and a stride of at least n");
     }
 
+    void* const ws = need ? reinterpret_cast<void*>(uintptr_t(256)) : d->workspace;
+    const int64_t ws_bytes = need ? (int64_t)1 << 60 : d->workspace_bytes;
     GemmParams p;
     memset(&p, 0, sizeof(p));
     const int64_t kalign = w4 ? 32 : 16;
@@ -196,14 +226,18 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
 
     if (groups && w4) {
         const int64_t kp = (kmax + 31) & ~(int64_t)31;
-        if (!d->workspace || !al(d->workspace, 16) || d->workspace_bytes < d->n * kp)
+        if (!ws || !al(ws, 16) || ws_bytes < d->n * kp)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors with int4 weights need %lld bytes of workspace",
                         (long long)(d->n * kp));
     }
-    if (w4 && d->workspace) {
+    if (w4 && ws) {
         // expand b to int8 in the caller's workspace and run the int8 kernels on it
         const int64_t kp = (kmax + 31) & ~(int64_t)31;  // whole 16-byte packed chunks
-        if (al(d->workspace, 16) && d->workspace_bytes >= d->batch * d->n * kp && kp / 2 <= d->ldb) {
+        if (al(ws, 16) && ws_bytes >= d->batch * d->n * kp && kp / 2 <= d->ldb) {
+            if (need) {
+                *need = d->batch * d->n * kp;
+                return SEGQ_OK;
+            }
             const int64_t chunks = kp / 32;
             for (int64_t zb = 0; zb < d->batch; ++zb) {
                 const int64_t total = d->n * chunks;
@@ -261,13 +295,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     }
     // int8 with several ranges keeps the big tiles if the caller lends a workspace to park
     // finished ranges in: one fp32 tile per workgroup
-    bool park = i8 && plain8 && fold && !groups && wide_ok && d->batch == 1 && d->out_dtype != SEGQ_ACC && d->workspace &&
-                al(d->workspace, 16);
+    bool park = i8 && plain8 && fold && !groups && wide_ok && d->batch == 1 && d->out_dtype != SEGQ_ACC && ws && al(ws, 16);
     auto park_fits = [&](int c) {
         if (c < FIRST_WIDE_CFG || c > FIRST_WIDE_CFG + 5) return false;
         const TileCfg& t = TILE_CFGS[c];
         const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
-        return d->workspace_bytes >= tiles * t.bm * t.bn * 4;
+        return ws_bytes >= tiles * t.bm * t.bn * 4;
     };
     if (d->tile == 0) {
         if (groups) {
@@ -290,8 +323,8 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     int splits = 1;
     int64_t part_bytes = 0;
     {
-        const bool can = plain8 && wide_ok && d->batch == 1 && !groups && d->out_dtype != SEGQ_ACC && d->workspace &&
-                         al(d->workspace, 16) && d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG);
+        const bool can = plain8 && wide_ok && d->batch == 1 && !groups && d->out_dtype != SEGQ_ACC && ws && al(ws, 16) &&
+                         d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG);
         const int64_t total_steps = ktotal / 128;
         if (d->split_k > 1 && !can)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: split_k needs plain 8-bit codes, K ranges in multiples of 128, one problem, "
@@ -311,8 +344,9 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
                 // 96 tiles x 2 shares lose to 192 tiles of 256 x 128 (4096 x 6144 x 1536): the fp32 partial
                 // results and their sum cost what two shares gain
                 // (int8 with several ranges gains nothing: 139 -> 145 us on the same shape)
-                if (tiles * 4 <= 256 && total_steps >= 32 && !(i8 && fold)) {
-                    const int64_t by_cus = 256 / tiles, by_steps = total_steps / 8;
+                const int64_t cus = device_cus();
+                if (tiles * 4 <= cus && total_steps >= 32 && !(i8 && fold)) {
+                    const int64_t by_cus = cus / tiles, by_steps = total_steps / 8;
                     want = (int)(by_cus < by_steps ? by_cus : by_steps);
                     if (want > 16) want = 16;
                 }
@@ -324,7 +358,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
                 const int64_t pb = (((int64_t)s_ * d->m * d->n * 4) + 255) & ~(int64_t)255;
                 return pb + (need_park || park ? (int64_t)s_ * tiles * t.bm * t.bn * 4 : 0);
             };
-            while (want > 1 && bytes_for(want) > d->workspace_bytes) --want;
+            while (want > 1 && bytes_for(want) > ws_bytes) --want;
             if (d->split_k > 1 && want < 2) return fail(SEGQ_ERR_ARG, "segq_gemm: workspace too small for split_k");
             if (want > 1) {
                 splits = want;
@@ -335,7 +369,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
         }
     }
     if (splits == 1 && d->tile != 0) park = park && park_fits(cfg);
-    if (park) p.park = reinterpret_cast<float*>(static_cast<uint8_t*>(d->workspace) + part_bytes);
+    if (park) p.park = reinterpret_cast<float*>(static_cast<uint8_t*>(ws) + part_bytes);
     if (park) {
         // every 8-wave tile serves several ranges this way
     } else if (cfg >= FIRST_WIDE_CFG) {
@@ -353,6 +387,10 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st) {
     const TileCfg& c = TILE_CFGS[cfg];
     p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);
     p.tiles_n = (int32_t)((d->n + c.bn - 1) / c.bn);
+    if (need) {
+        *need = part_bytes + (park ? (int64_t)splits * p.tiles_m * p.tiles_n * c.bm * c.bn * 4 : 0);
+        return SEGQ_OK;
+    }
     p.group_m = 8;
     if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff || d->batch > 65535) return fail(SEGQ_ERR_ARG, "segq_gemm: grid too large");
     const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
@@ -431,9 +469,37 @@ int segq_gemm(const segq_gemm_desc* d, segq_stream_t stream) { return gemm_impl(
 
 int segq_gemm_tile_count(void) { return NUM_TILE_CFG; }
 
+int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes) {
+    if (!bytes) return fail(SEGQ_ERR_ARG, "segq_gemm_workspace_bytes: null result pointer");
+    return gemm_impl(d, nullptr, bytes);
+}
+
 int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream) {
     if (!q || !g) return fail(SEGQ_ERR_ARG, "segq_linear: null descriptor");
+    // the GEMM must consume exactly what the quantise step produces
     if (q->codes != g->a) return fail(SEGQ_ERR_ARG, "segq_linear: the GEMM must read the codes the quantise step writes");
+    if (g->n_ranges < 1 || g->n_ranges > SEGQ_MAX_RANGES) return fail(SEGQ_ERR_ARG, "segq_linear: n_ranges %d out of range", g->n_ranges);
+    bool reads_neg = false;
+    for (int i = 0; i < g->n_ranges; ++i) reads_neg = reads_neg || g->ranges[i].a_sel == 1;
+    if (reads_neg && (!q->codes_neg || q->codes_neg != g->a_neg))
+        return fail(SEGQ_ERR_ARG, "segq_linear: a range reads a_neg, which is not the second code tensor the quantise step writes");
+    if (q->ld_codes != g->lda || q->rows != g->m * g->batch)
+        return fail(SEGQ_ERR_ARG, "segq_linear: the code tensor's rows (%lld, stride %lld) do not match the GEMM's (%lld, stride %lld)",
+                    (long long)q->rows, (long long)q->ld_codes, (long long)(g->m * g->batch), (long long)g->lda);
+    if (q->code_fmt != g->a_fmt) return fail(SEGQ_ERR_ARG, "segq_linear: code formats differ (%d written, %d read)", q->code_fmt, g->a_fmt);
+    if (q->dynamic && g->out_dtype != SEGQ_ACC) {
+        // dynamic scales are outputs of the first step: every range must divide by one of them
+        const int64_t seg_rows = q->seg_rows > 0 ? q->seg_rows : q->rows;
+        const int64_t extent = (seg_rows > 0 ? (q->rows - 1) / seg_rows : 0) * q->seg_stride + (seg_rows - 1) * q->row_stride +
+                               (int64_t)(q->n_kseg - 1) * q->kseg_stride + 1;
+        for (int i = 0; i < g->n_ranges; ++i) {
+            const float* sx = g->ranges[i].sx;
+            const bool in_pos = q->scale && sx >= q->scale && sx < q->scale + extent;
+            const bool in_neg = q->scale_neg && sx >= q->scale_neg && sx < q->scale_neg + extent;
+            if (!in_pos && !in_neg)
+                return fail(SEGQ_ERR_ARG, "segq_linear: range %d divides by scales the dynamic quantise step does not write", i);
+        }
+    }
     const int rc = quantize_impl(q, static_cast<hipStream_t>(stream), nullptr);
     if (rc != SEGQ_OK) return rc;
     return gemm_impl(g, static_cast<hipStream_t>(stream));

@@ -16,6 +16,13 @@ int fail(int status, const char* fmt, ...);
 // Checks the launch that was just enqueued.
 int check_launch(const char* what);
 
+// Compute units of the current device (read once per device).
+int device_cus();
+
+// hipFuncAttributeMaxDynamicSharedMemorySize for `kern`, set once per kernel and
+// device: `done` is the kernel's own flag word, one bit per device ordinal.
+int reserve_lds(const void* kern, int bytes, unsigned long long* done);
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));

@@ -435,7 +435,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
 // ---- host-side launch of one (format, tile, fold) instance -------------------
 struct TileCfg { int bm, bn, wgm, wgn; };
 constexpr int NUM_TILE_CFG = 16;
-constexpr int FIRST_BIG_CFG = 8;    // two ids: the 4-wave 256 x 256 kernel (segq_gemm_big.h)
+constexpr int FIRST_BIG_CFG = 8;    // two retired ids (a 4-wave 256 x 256 kernel that no shape profited from)
 constexpr int FIRST_WIDE_CFG = 10;  // six ids: the 8-wave kernels (segq_gemm_wide.h); the last two plain int8 only
 constexpr TileCfg TILE_CFGS[NUM_TILE_CFG] = {
     {256, 256, 2, 2}, {256, 128, 2, 2}, {128, 128, 2, 2}, {64, 128, 2, 2}, {128, 256, 2, 2},
@@ -447,19 +447,13 @@ template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
 int launch_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_kernel<BM, BN, WGM, WGN, FMT, B4, FOLD>;
     constexpr int lds = 2 * (BM + BN) * BK;
-    static bool attr_set = false;  // one attribute call per kernel and process
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", lds);
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(WGM * WGN * 64), lds, st, p);
     return check_launch("segq_gemm");
 }
 
-template <int FMT, bool DIRECT>
-int launch_big(const GemmParams& p, int64_t batch, hipStream_t st);
 template <int FMT, bool B4>
 int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st);
 
@@ -470,10 +464,8 @@ int launch_format(const GemmParams& p, int cfg, bool fold, int64_t batch, hipStr
         for (int i = 0; i < p.nr; ++i) asel = asel || p.r[i].a_sel >= 2;
         return launch_wide<FMT, B4>(p, cfg - FIRST_WIDE_CFG, fold, asel, batch, st);
     }
-    if constexpr (!B4) {
-        if (!fold && cfg == FIRST_BIG_CFG) return launch_big<FMT, false>(p, batch, st);
-        if (!fold && cfg == FIRST_BIG_CFG + 1) return launch_big<FMT, true>(p, batch, st);
-    }
+    if (cfg == FIRST_BIG_CFG || cfg == FIRST_BIG_CFG + 1)
+        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile ids %d and %d are retired", FIRST_BIG_CFG + 1, FIRST_BIG_CFG + 2);
     switch (cfg * 2 + (fold ? 1 : 0)) {
         case 0: return launch_instance<256, 256, 2, 2, FMT, B4, false>(p, batch, st);
         case 2: return launch_instance<256, 128, 2, 2, FMT, B4, false>(p, batch, st);

@@ -17,9 +17,46 @@
 //    16 lines per instruction (measured 1.7 TB/s); transposed through a private
 //    LDS patch every store instruction writes four full 256-byte row pieces.
 #pragma once
-#include "segq_gemm_big.h"
+#include "segq_gemm_kernel.h"
+#include <type_traits>
 
 namespace segq {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+// One lane's 16 bytes from global memory to LDS at lds_base + lane * 16.
+__device__ __forceinline__ void load16_to_lds(const uint8_t* g, uint8_t* lds_base) {
+    __builtin_amdgcn_global_load_lds((glb_ptr_t)g, (lds_ptr_t)lds_base, 16, 0, 0);
+}
+
+// Four consecutive outputs of one row, rounded once to the output type.
+template <int OUT>
+__device__ __forceinline__ void store4(void* C, int64_t e, const float (&o)[4], bool vec, int n_left) {
+    if constexpr (OUT == SEGQ_F32) {
+        float* dst = static_cast<float*>(C) + e;
+        if (vec) {
+            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (v < n_left) dst[v] = o[v];
+        }
+    } else {
+        const uint32_t lo = (OUT == SEGQ_BF16) ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]);
+        const uint32_t hi = (OUT == SEGQ_BF16) ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]);
+        uint16_t* dst = static_cast<uint16_t*>(C) + e;
+        if (vec) {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        } else {
+            const uint32_t h[4] = {lo & 0xffffu, lo >> 16, hi & 0xffffu, hi >> 16};
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (v < n_left) dst[v] = (uint16_t)h[v];
+        }
+    }
+}
+
 
 // Scale, add bias, round once, store.  16-bit outputs of full tiles go through a
 // per-wave LDS patch so that every store instruction writes whole row pieces.
@@ -1020,12 +1057,8 @@ template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool AS
 int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_wide_kernel<BM, BN, WGM, WGN, FMT, B4, FOLD, ASEL>;
     constexpr int lds = 2 * (BM + BN) * BK;
-    static bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", lds);
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(WGM * WGN * 64), lds, st, p);
     return check_launch("segq_gemm");
@@ -1037,12 +1070,8 @@ int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK>;
     // the stages, the epilogue's vectors, and the ring of group factors
     constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4 + (GRP ? 4 * BN * 4 : 0);
-    static bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return fail(SEGQ_ERR_LAUNCH, "segq_gemm: cannot reserve %d bytes of LDS", lds);
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(WGM * WGN * 64), lds, st, p);
     return check_launch("segq_gemm");

@@ -183,7 +183,7 @@ class SegmentLinear(nn.Module):
         the output) are the hooks for the reference's SmoothQuant division and SVD low-rank
         branch (segquant/optimum/optimizer.py:467-470, :731-740), fused into the same kernels."""
         opt = self.optimizer
-        if not chunked and opt.real_quant and opt.has_calibrated:
+        if not chunked and opt.fused_available():
             return opt.forward_fused(x, self.bias_data if self.bias else None, pre_op=pre_op, gate=gate,
                                      col_div=col_div, addend=addend)
         if pre_op is not None:

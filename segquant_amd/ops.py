@@ -99,16 +99,26 @@ def code_dtype(fmt: str) -> torch.dtype:
 # ---------------------------------------------------------------------------
 # quantise
 # ---------------------------------------------------------------------------
-def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional[torch.Tensor] = None, *,
+def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional[torch.Tensor] = None, **kw):
+    """Quantise a 2-D float matrix ``x`` (rows, cols) to codes: :func:`quantize_desc` + one
+    ``segq_quantize`` launch.  Returns the code tensor, or ``(Xp, Xn)`` when ``two_tensors``."""
+    d, result, info, _keep = quantize_desc(x, fmt, scale, scale_neg, **kw)
+    L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
+    return result
+
+
+def quantize_desc(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional[torch.Tensor] = None, *,
              seg_rows: int = 0, seg_stride: int = 0, row_stride: int = 0,
              kseg_bounds: Optional[Sequence[int]] = None, kseg_stride: int = 0,
              dual: bool = False, dual_kseg_mask: int = 0xFFFFFFFF, dynamic: bool = False,
              two_tensors: bool = False, out: Optional[torch.Tensor] = None,
              out_neg: Optional[torch.Tensor] = None, pre_op: Optional[str] = None,
              gate: Optional[torch.Tensor] = None, col_div: Optional[torch.Tensor] = None):
-    """Quantise a 2-D float matrix ``x`` (rows, cols) to codes.
+    """The ``segq_quant_desc`` of a quantise launch, its output tensor(s), the launch's
+    description for ``record_launches`` and the tensors the descriptor points into
+    (keep them alive until the launch is enqueued).
 
-    See ``segq_quantize`` in include/segq.h for the scale indexing.  Returns the
+    See ``segq_quantize`` in include/segq.h for the scale indexing.  The result is the
     code tensor, or ``(Xp, Xn)`` when ``two_tensors`` (DualScale in the
     reference's two-tensor layout).  With ``dynamic`` the scale tensors are
     written by the kernel.  ``pre_op`` ("gelu_tanh", "gelu", "silu") fuses the
@@ -161,8 +171,7 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
         d.gate = gate.data_ptr(); d.ld_gate = gate.stride(0) if rows > 1 else cols
     info = dict(rows=rows, cols=cols, x_bytes=x.element_size() * (2 if gate is not None else 1),
                 code_bytes=0.5 if fmt == FMT_INT4 else 1.0, tensors=2 if two_tensors else 1, dynamic=bool(dynamic))
-    L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
-    return (out, out_neg) if two_tensors else out
+    return d, ((out, out_neg) if two_tensors else out), info, (x, scale, scale_neg, gate, col_div, out, out_neg)
 
 
 # ---------------------------------------------------------------------------
@@ -181,19 +190,45 @@ class Range:
 
 
 _int4_ws = {}
+_retired_ws = []  # outgrown buffers stay allocated: a captured HIP graph may still hold their address
 
 
 def int4_workspace(device, nbytes: int) -> torch.Tensor:
-    """A per-device scratch tensor of at least ``nbytes`` for ``gemm``'s ``workspace``
-    (expanded int4 weights, or the parked partial sums of int8 ranges), grown on demand
-    and shared by every layer (launches on one stream run in order, and its contents
-    only live for the duration of one GEMM launch)."""
-    key = torch.device(device)
+    """A scratch tensor of at least ``nbytes`` for ``gemm``'s ``workspace`` (expanded int4
+    weights, parked partial sums of int8 ranges, split-K partial results), one per device
+    and stream: launches on one stream run in order and the contents only live for the
+    duration of one GEMM launch, so every layer on that stream can share it.  Grown on
+    demand; a buffer that was handed out is never freed."""
+    dev = torch.device(device)
+    if dev.index is None:
+        dev = torch.device(dev.type, torch.cuda.current_device())
+    key = (dev, torch.cuda.current_stream(dev).cuda_stream)
     ws = _int4_ws.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=key)
+        if ws is not None:
+            _retired_ws.append(ws)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         _int4_ws[key] = ws
     return ws
+
+
+def gemm_workspace_bytes(g) -> int:
+    """Workspace the launch described by ``g`` (the tuple :func:`gemm_desc` returns) would use if it
+    were lent as much as the library can make use of; 0 if it has no use for one
+    (``segq_gemm_workspace_bytes``)."""
+    n = C.c_int64(0)
+    L.check(L.lib().segq_gemm_workspace_bytes(C.byref(g[0]), C.byref(n)))
+    return n.value
+
+
+def gemm_launch(g, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Enqueue the GEMM described by ``g``, lending it ``workspace`` (a byte tensor) if given."""
+    d, out, info, _keep = g
+    if workspace is not None:
+        _need_cuda(workspace)
+        d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()
+    L.check(_launch("gemm", info, lambda: L.lib().segq_gemm(C.byref(d), _stream())))
+    return out
 
 
 def park_bytes(m: int, n: int) -> int:
@@ -218,14 +253,33 @@ def auto_splits(m: int, n: int, k_steps: int) -> int:
     return max(0, min(256 // tiles, k_steps // 8, 16))
 
 
-def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
+def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], **kw) -> torch.Tensor:
+    """Segmented GEMM with fused de-quantisation and bias: :func:`gemm_desc` + one ``segq_gemm`` call."""
+    d, out, info, _keep = gemm_desc(a, b, ranges, **kw)
+    L.check(_launch("gemm", info, lambda: L.lib().segq_gemm(C.byref(d), _stream())))
+    return out
+
+
+def linear(q, g) -> torch.Tensor:
+    """``segq_linear``: the quantise launch described by ``q`` and the GEMM described by ``g`` (the
+    tuples :func:`quantize_desc` and :func:`gemm_desc` return) in one call of the library.  The GEMM
+    must read the code tensor(s) the quantise step writes, and with dynamic scales the scale
+    tensors it fills."""
+    qd, _codes, qinfo, _k1 = q
+    gd, out, ginfo, _k2 = g
+    L.check(_launch("linear", dict(q=qinfo, g=ginfo), lambda: L.lib().segq_linear(C.byref(qd), C.byref(gd), _stream())))
+    return out
+
+
+def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n: int, a_fmt: str, b_fmt: str,
          out_dtype, lda: int, ldb: int, a_neg: Optional[torch.Tensor] = None,
          bias: Optional[torch.Tensor] = None, batch: int = 1, batch_stride_a: int = 0, batch_stride_b: int = 0,
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
          tile: int = 0, workspace: Optional[torch.Tensor] = None,
          group_dequant: Optional[torch.Tensor] = None, split_k: int = 0,
-         addend: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Segmented GEMM with fused de-quantisation and bias (``segq_gemm``).
+         addend: Optional[torch.Tensor] = None):
+    """The ``segq_gemm_desc`` of a segmented GEMM with fused de-quantisation and bias, its output
+    tensor, the launch's description and the tensors the descriptor points into.
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
     accumulators (int32 for integer codes, float32 for e4m3).  ``workspace``: a
@@ -281,8 +335,7 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: int, n
         kr.sw = r.sw.data_ptr() if r.sw is not None else None
     info = dict(m=m, n=n, batch=batch, k_alg=sum(r.k_len for r in ranges if r.a_sel in (0, 2)),
                 k_exec=sum(r.k_len for r in ranges), a_fmt=a_fmt, b_fmt=b_fmt)
-    L.check(_launch("gemm", info, lambda: L.lib().segq_gemm(C.byref(d), _stream())))
-    return out
+    return d, out, info, (a, b, a_neg, bias, workspace, group_dequant, addend, out, list(ranges))
 
 
 # ---------------------------------------------------------------------------

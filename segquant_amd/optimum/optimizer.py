@@ -209,7 +209,11 @@ class DefaultOptimizer(BaseOptimizer):
 
     # ---- the fused route -------------------------------------------------
     def fused_available(self) -> bool:
-        return self.real_quant and self.has_calibrated
+        """The one-launch route serves up to SEGQ_MAX_KSEG input segments; layers with more
+        (the reference accepts any number of equal chunks) take the reference-convention
+        operator, one batched launch over the segments."""
+        few = self.seg_mode != "input" or self.chunks <= ops.L.SEGQ_MAX_KSEG
+        return bool(self.real_quant and self.has_calibrated and few)
 
     def _build_plan(self, device):
         """Turns segments and calibrated scales into what the kernels take."""
@@ -320,25 +324,30 @@ class DefaultOptimizer(BaseOptimizer):
             else:
                 ranges.append(ops.Range(k0, k1 - k0, pos[s], plan["sw"], 0, rs, plan["sw_cs"]))
         ldb = K // 2 if plan["fw"] == ops.FMT_INT4 else K
-        # int4 weights and many tokens: the GEMM is bound by the matrix cores, so lend the
-        # library N x K bytes to expand the weights into once per launch (the int8 kernels
-        # then run); with few tokens reading half the weight bytes matters more
-        # (measured, K 1280, N 10240: 161 -> 119 us at 8192 tokens, no gain at 2048)
-        # (group-wise scales run on the int8 kernels only: always lend)
         gdq = plan.get("group_dequant")
-        ws = ops.int4_workspace(x.device, N * K) if plan["fw"] == ops.FMT_INT4 and (M >= 3072 or gdq is not None) else None
-        # int8 with several ranges (K segments, DualScale) and many tokens: lend room to park the
-        # finished ranges' sums, which keeps the big tiles (4608 x 15360 x 3072, three ranges:
-        # 441 -> 383 us; 9216 tokens: 1044 -> 756 us; no gain at 1024 tokens)
-        if ws is None and gdq is None and plan["fa"] == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1 and M >= 2048:
-            ws = ops.int4_workspace(x.device, ops.park_bytes(M, N))
-        # few tiles, long K (config 5 at 1024 tokens): room for the library to share the K steps of a
-        # tile between workgroups (it does for e4m3 and for single-range int8)
-        if ws is None and gdq is None and plan["fw"] != ops.FMT_INT4:
-            ns = ops.auto_splits(M, N, sum(r.k_len for r in ranges) // 128)
-            if ns > 1:
-                ws = ops.int4_workspace(x.device, ops.split_bytes(M, N, ns))
-        out = ops.gemm(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
-                       lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, workspace=ws, group_dequant=gdq,
-                       addend=None if addend is None else addend.reshape(M, N).contiguous())
+        g = ops.gemm_desc(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
+                          lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, group_dequant=gdq,
+                          addend=None if addend is None else addend.reshape(M, N).contiguous())
+        # Whether to lend the library a workspace is this layer's call; how much it could use is
+        # the library's (segq_gemm_workspace_bytes), asked once per token count.
+        #  * int4 weights and many tokens: the GEMM is bound by the matrix cores, so the weights are
+        #    expanded to int8 once per launch and the int8 kernels run; with few tokens reading half
+        #    the weight bytes matters more (measured, K 1280, N 10240: 161 -> 119 us at 8192 tokens,
+        #    no gain at 2048).  Group-wise scales run on the int8 kernels only: always lend.
+        #  * int8 with several ranges (K segments, DualScale) and many tokens: room to park the
+        #    finished ranges' sums keeps the big tiles (4608 x 15360 x 3072, three ranges:
+        #    441 -> 383 us; 9216 tokens: 1044 -> 756 us; no gain at 1024 tokens).
+        #  * few tiles and a long K (config 5 at 1024 tokens): room to share the K steps of a tile
+        #    between workgroups.
+        int4 = plan["fw"] == ops.FMT_INT4
+        int8_ranges = plan["fa"] == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1
+        lend = (M >= 3072 or gdq is not None) if int4 else (M >= 2048 or not int8_ranges)
+        ws = None
+        if lend:
+            need = plan.setdefault("ws_need", {}).get(M)
+            if need is None:
+                need = plan["ws_need"][M] = ops.gemm_workspace_bytes(g)
+            if need:
+                ws = ops.int4_workspace(x.device, need)
+        out = ops.gemm_launch(g, ws)
         return out.view(*x.shape[:-1], N)

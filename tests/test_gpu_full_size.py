@@ -169,25 +169,109 @@ def test_full_size_group_wise_scales_product_check(ops, M, K, N):
     assert np.abs(l @ c - left).max() <= 2e-6 * max(np.abs(left).max(), np.sqrt(M) * np.abs(c).max())
 
 
-@pytest.mark.parametrize("M", [1024, 4608])
+def _bands(M, N):
+    """Rows and columns on the borders of every tile size the library picks (128, 192, 256, 288),
+    the first and last ones, and a few in the middle."""
+    rows = sorted({r for r in (0, 1, 15, 16, 127, 128, 191, 192, 255, 256, 287, 288, M // 2, M // 2 + 1, M - 289, M - 257,
+                               M - 193, M - 129, M - 2, M - 1) if 0 <= r < M})
+    cols = sorted({c for c in (0, 1, 3, 4, 127, 128, 191, 192, 255, 256, 287, 288, N // 2 + 5, N - 289, N - 257, N - 193,
+                               N - 129, N - 2, N - 1) if 0 <= c < N})
+    return rows, cols
+
+
+@pytest.mark.parametrize("M", [1024, 4608, 9216])
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
-def test_full_size_config5_ranges_parked_or_split(ops, M, fmt):
-    """Configuration 5 (K = 3072 | 12288, the second segment read from two code tensors) with the
-    workspace the layer lends: int8 parks its finished ranges, 1024 tokens of e4m3 share the K
-    steps of a tile between workgroups.  Same answer as the launch without a workspace (second
-    accumulator set / in-place rescaling, one workgroup per tile), to fp32 summation order."""
+@pytest.mark.parametrize("lend", [False, True])
+def test_full_size_config5_three_ranges_against_closed_form(ops, M, fmt, lend):
+    """Configuration 5 (K = 3072 | 12288, the second segment read from two code tensors, per-token
+    scales on it) at every M of the sweep, the library choosing tile and split (tile = 0): with the
+    workspace the layer lends (int8 parks its finished ranges, few tokens share the K steps of a
+    tile between workgroups) and without (second accumulator set / fp32 sums rescaled in place).
+    Row and column bands of the fp32 output against the fp64 closed form
+    sum_r A_r B_r^T / (sx_r sw) + bias (segquant/src/real_quant/dequantizer.cuh:53-74 for the
+    two halves of the DualScale segment, real_gemm.cu:752-894)."""
     K0, K1, N = 3072, 12288, 3072
     K = K0 + K1
     a, a2, b = _codes((M, K), fmt, 130), _codes((M, K), fmt, 131), _codes((N, K), fmt, 132)
     ad, a2d, bd = _dev(a, fmt), _dev(a2, fmt), _dev(b, fmt)
     g = torch.Generator().manual_seed(133)
-    s0 = (torch.rand(1, generator=g) + 0.5).to(DEV)
-    sx, sx2 = (torch.rand(M, generator=g) + 0.5).to(DEV), (torch.rand(M, generator=g) + 0.5).to(DEV)
-    sw, bias = (torch.rand(N, generator=g) + 0.5).to(DEV), torch.randn(N, generator=g).to(DEV)
-    rg = [ops.Range(0, K0, s0, sw, 0, 0, 1), ops.Range(K0, K1, sx, sw, 0, 1, 1), ops.Range(K0, K1, sx2, sw, 1, 1, 1)]
-    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, bias=bias, a_neg=a2d)
-    plain = ops.gemm(ad, bd, rg, split_k=1, **kw)
-    nbytes = max(ops.park_bytes(M, N), ops.split_bytes(M, N, max(ops.auto_splits(M, N, (K0 + 2 * K1) // 128), 1)))
-    lent = ops.gemm(ad, bd, rg, workspace=torch.empty(nbytes, dtype=torch.uint8, device=DEV), **kw)
-    tol = 3e-6 if fmt == O.FMT_INT8 else 2e-4
-    assert (lent - plain).abs().max().item() <= tol * plain.abs().max().item()
+    s0 = torch.rand(1, generator=g) + 0.5
+    sx, sx2 = torch.rand(M, generator=g) + 0.5, torch.rand(M, generator=g) + 0.5
+    sw, bias = torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    s0d, sxd, sx2d, swd = (t.to(DEV) for t in (s0, sx, sx2, sw))
+    rg = [ops.Range(0, K0, s0d, swd, 0, 0, 1), ops.Range(K0, K1, sxd, swd, 0, 1, 1), ops.Range(K0, K1, sx2d, swd, 1, 1, 1)]
+    ws = None
+    if lend:
+        nbytes = max(ops.park_bytes(M, N), ops.split_bytes(M, N, max(ops.auto_splits(M, N, (K0 + 2 * K1) // 128), 1)))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    out = ops.gemm(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, bias=bias.to(DEV),
+                   a_neg=a2d, workspace=ws)
+    got = out.cpu().numpy().astype(np.float64)
+    av, a2v, bv = O.code_values(a, fmt), O.code_values(a2, fmt), O.code_values(b, fmt)
+    s0n, sxn, sx2n, swn, bn = (t.numpy().astype(np.float64) for t in (s0, sx, sx2, sw, bias))
+
+    def check(ri, ci):
+        A0, A1, A2 = av[ri][:, :K0], av[ri][:, K0:], a2v[ri][:, K0:]
+        B0, B1 = bv[ci][:, :K0], bv[ci][:, K0:]
+        d0 = s0n[0] * swn[ci][None, :]
+        d1 = sxn[ri][:, None] * swn[ci][None, :]
+        d2 = sx2n[ri][:, None] * swn[ci][None, :]
+        t0, t1, t2 = (A0 @ B0.T) / d0, (A1 @ B1.T) / d1, (A2 @ B1.T) / d2
+        want = t0 + t1 + t2 + bn[ci][None, :]
+        terms = np.abs(t0) + np.abs(t1) + np.abs(t2) + np.abs(bn[ci])[None, :]
+        err = np.abs(got[np.ix_(ri, ci)] - want)
+        # element-wise.  Integer sums are exact, so what is left is fp32 rounding of each term (a
+        # hardware reciprocal and two products) and of their sum: a few ulp of the terms' sizes.
+        # e4m3: the MFMA adds each 128-long group with a limited-width adder, 2e-4 of sum |a||b|.
+        bound = 2e-6 * terms
+        if fmt == O.FMT_E4M3:
+            bound = bound + 2e-4 * ((np.abs(A0) @ np.abs(B0).T) / d0 + (np.abs(A1) @ np.abs(B1).T) / d1 +
+                                    (np.abs(A2) @ np.abs(B1).T) / d2)
+        assert (err <= bound).all(), float((err / bound).max())
+
+    rows, cols = _bands(M, N)
+    check(np.asarray(rows), np.arange(N))
+    check(np.arange(M), np.asarray(cols))
+
+
+LAYER_CASES = [(1, None, torch.float32), (2, None, torch.bfloat16), (5, 9216, torch.bfloat16), (5, 1024, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("config,M,dtype", LAYER_CASES)
+def test_full_size_layers_against_the_oracle(config, M, dtype):
+    """SegmentLinear at the benchmark's own sizes with the library's own tile choice and the layer's
+    own workspace lending: configuration 1 (256 tokens, whole output), configuration 2 (4096 tokens:
+    fc1 on the two-workgroup 128 x 128 kernel, fc2 DualScale in two code tensors) and configuration 5
+    at 9216 and 1024 tokens (int8 parked, e4m3 rescaled in place, split K), on row and column bands
+    against the closed form built by the oracle from the layer's codes and scales
+    (element-wise: one rounding to the output dtype plus the accumulation's own error)."""
+    from _layer_oracle import _np32, oracle_layer_output
+    from segquant_amd import workloads as W
+    for spec in W.config_linears(config, M=M):
+        layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+        assert layer.optimizer.real_quant, spec.name
+        xin = x.to(spec.x_dtype).to(DEV)
+        out = layer(xin)
+        assert out.shape == (spec.M, spec.N) and out.dtype == spec.x_dtype
+        got = _np32(out).astype(np.float64)
+        x_np = _np32(xin)
+        del xin, out
+        fp8 = spec.act == O.FMT_E4M3
+        ulp = {torch.float32: 2.0 ** -22, torch.bfloat16: 2.0 ** -8}[spec.x_dtype]
+        rows, cols = _bands(spec.M, spec.N)
+        if spec.M * spec.N * spec.K <= 2 ** 33:
+            bands = [(None, None)]
+        else:
+            bands = [(rows, None), (None, cols)]
+        for ri, ci in bands:
+            want = oracle_layer_output(layer, spec, x_np, rows=ri, cols=ci)
+            sub = got if ri is None and ci is None else got[np.ix_(np.arange(spec.M) if ri is None else ri,
+                                                                   np.arange(spec.N) if ci is None else ci)]
+            scale = np.abs(want).max()
+            # one rounding of the output, plus the accumulation error measured against the largest output
+            # (sums of K-range terms that cancel): fp32 for integer codes, the MFMA's summation for e4m3
+            bound = ulp * np.abs(want) + (1e-3 if fp8 else 2e-6) * scale
+            err = np.abs(sub - want)
+            assert (err <= bound).all(), (spec.name, float((err / bound).max()))
+        del layer
+        torch.cuda.empty_cache()

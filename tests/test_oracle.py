@@ -379,3 +379,44 @@ def test_smooth_divide_is_torchs_in_place_division(dt):
     s = torch.rand(96, generator=g) * 3 + 0.01
     want = x.clone().div_(s.to(tdt)).float().numpy()
     assert np.array_equal(O.smooth_divide(x.float().numpy(), s.numpy(), dt), want)
+
+
+def test_dequant_dual_against_fp64_closed_form_and_reductions():
+    """dequant_dual (segquant/src/real_quant/dequantizer.cuh:53-74) pinned without reference to its
+    own formula's code: (a) the fp64 value Yp/(pos sw) + Yn/(neg sw) written out with explicit
+    per-token / per-channel indices, to fp32 rounding; (b) with power-of-two scales every fp32
+    operation is exact, so the result must equal the fp64 value bit for bit; (c) Yn = 0 reduces it
+    to the single-scale dequant, and pos == neg to the dequant of Yp + Yn."""
+    g = np.random.default_rng(11)
+    S, M, N = 2, 5, 7  # all different: a transposed or mis-broadcast scale changes the result
+    yp = g.integers(0, 3_000_000, size=(S, M, N)).astype(np.int32)
+    yn = -g.integers(0, 3_000_000, size=(S, M, N)).astype(np.int32)
+    for per_tok in (False, True):
+        for per_ch in (False, True):
+            pos = (g.random(S * M if per_tok else S) * 30 + 1).astype(np.float32)
+            neg = (g.random(S * M if per_tok else S) * 60 + 1).astype(np.float32)
+            sw = (g.random(S * N if per_ch else S) * 50 + 1).astype(np.float32)
+            got = O.dequant_dual(yp, yn, pos, neg, sw)
+            want = np.empty((S, M, N))
+            for s in range(S):
+                for m in range(M):
+                    for n in range(N):
+                        p = np.float64(pos[s * M + m] if per_tok else pos[s])
+                        q = np.float64(neg[s * M + m] if per_tok else neg[s])
+                        w = np.float64(sw[s * N + n] if per_ch else sw[s])
+                        want[s, m, n] = yp[s, m, n] / (p * w) + yn[s, m, n] / (q * w)
+            size = np.abs(yp / 1.0) + np.abs(yn / 1.0)
+            assert got.dtype == np.float32
+            assert (np.abs(got - want) <= 4 * 2.0 ** -24 * np.maximum(np.abs(want), size / 31.0)).all()
+    # (b) exact arithmetic
+    pos = np.float32([2.0, 8.0]); neg = np.float32([4.0, 0.5]); sw = np.float32([16.0, 2.0])
+    yp2 = (yp >> 8).astype(np.int32); yn2 = -((-yn) >> 8).astype(np.int32)  # below 2^24: exact as fp32
+    got = O.dequant_dual(yp2, yn2, pos, neg, sw)
+    want = yp2 / (pos.astype(np.float64) * sw)[:, None, None] + yn2 / (neg.astype(np.float64) * sw)[:, None, None]
+    assert np.array_equal(got.astype(np.float64), want.astype(np.float32).astype(np.float64))
+    # bf16 output: one rounding of that sum
+    got_bf = O.dequant_dual(yp2, yn2, pos, neg, sw, "bf16")
+    assert np.array_equal(got_bf, O.round_to_bf16(want.astype(np.float32)))
+    # (c) reductions
+    assert np.array_equal(O.dequant_dual(yp2, np.zeros_like(yp2), pos, neg, sw), O.dequant(yp2, pos, sw))
+    assert np.array_equal(O.dequant_dual(yp2, yn2, pos, pos, sw), O.dequant(yp2 + yn2, pos, sw))
