@@ -256,6 +256,34 @@ int segq_gemm_tile_count(void);
  * allocates its temporaries itself (segquant/src/real_quant/real_gemm.cu:684-698, :855-865). */
 int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes);
 
+/* ------------------------------------------------------------------------
+ * segq_gemm for callers that cannot allocate device memory.
+ *
+ * No counterpart in the reference (whose operators allocate every temporary through ATen,
+ * segquant/src/real_quant/real_gemm.cu:684-698).  It is for callers that cannot call hipMalloc or an
+ * allocating framework routine around the launch: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation.  Same descriptor, same kernels and same result as
+ * segq_gemm called with a workspace of segq_gemm_workspace_bytes(d) bytes, but the workspace
+ * (expanded int4 weights, parked sums of int8 ranges, split-K partial results) is an array of
+ * SEGQ_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, from the
+ * first use on that GPU until the process ends; d->workspace is ignored.  A launch that would
+ * use more than that is refused with SEGQ_ERR_ARG and a message (nothing is enqueued).  The call
+ * allocates nothing and frees nothing; the array's address on the current device is resolved on
+ * the first call there, or ahead of time by segq_init().
+ *
+ * All calls on one GPU share that GPU's array and its contents are undefined between calls
+ * (nothing in it needs to start at zero: every kernel writes a slot before it reads it), so two
+ * such calls must not overlap on one GPU: issue them on one stream, or order the streams.
+ * ---------------------------------------------------------------------- */
+#define SEGQ_NOALLOC_SCRATCH_BYTES (64ll << 20)
+int segq_gemm_noalloc(const segq_gemm_desc* d, segq_stream_t stream);
+int64_t segq_noalloc_scratch_bytes(void); /* SEGQ_NOALLOC_SCRATCH_BYTES of the loaded library */
+
+/* Optional set-up for the current device, outside any stream capture: reads the device's
+ * properties and resolves the scratch array's address there, which the entry points otherwise do
+ * on their first call on that device.  No counterpart in the reference. */
+int segq_init(void);
+
 /* Quantise-then-multiply in one call: q writes its codes into a caller-provided
  * workspace that g reads as its a (and a_neg).  Replaces the body of
  * real_quantized_gemm_scaled / real_quantized_gemm_dual_scaled

@@ -425,6 +425,29 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, int64_t* need = nu
     return launch_gemm_w4(p, cfg, fold, d->batch, st);
 }
 
+// ---- the library's own scratch memory, for segq_gemm_noalloc -------------------------------
+// One array per GPU the library runs on, held until the process ends.  In host code the name
+// `scratch` is only a handle for hipGetSymbolAddress: the device address it resolves to (one per
+// device, each GPU holding its own copy) is what kernels, copies and fills are given.
+constexpr int64_t SCRATCH_BYTES = SEGQ_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+static void* g_scratch_ptr[64];  // resolved address per device ordinal
+
+static int scratch_address(void** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return fail(SEGQ_ERR_LAUNCH, "segq: cannot tell the current device (or its ordinal is above 63)");
+    void* ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!ptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(SEGQ_ERR_LAUNCH, "segq: cannot resolve the scratch array on device %d: %s", dev, hipGetErrorString(e));
+        __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+    }
+    *out = ptr;
+    return SEGQ_OK;
+}
+
 }  // namespace segq
 
 using namespace segq;
@@ -472,6 +495,35 @@ int segq_gemm_tile_count(void) { return NUM_TILE_CFG; }
 int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes) {
     if (!bytes) return fail(SEGQ_ERR_ARG, "segq_gemm_workspace_bytes: null result pointer");
     return gemm_impl(d, nullptr, bytes);
+}
+
+int segq_init(void) {
+    void* ptr = nullptr;
+    (void)device_cus();
+    return scratch_address(&ptr);
+}
+
+int64_t segq_noalloc_scratch_bytes(void) { return SCRATCH_BYTES; }
+
+int segq_gemm_noalloc(const segq_gemm_desc* d, segq_stream_t stream) {
+    int64_t need = 0;
+    int rc = gemm_impl(d, nullptr, &need);
+    if (rc != SEGQ_OK) return rc;
+    if (need > SCRATCH_BYTES)
+        return fail(SEGQ_ERR_ARG, "segq_gemm_noalloc: this launch would use %lld bytes of workspace, the library's scratch "
+                                  "array holds %lld; use segq_gemm with a workspace of the caller's",
+                    (long long)need, (long long)SCRATCH_BYTES);
+    segq_gemm_desc c = *d;
+    c.workspace = nullptr;
+    c.workspace_bytes = 0;
+    if (need > 0) {
+        void* ptr = nullptr;
+        rc = scratch_address(&ptr);  // resolved once per device (segq_init does it ahead of time)
+        if (rc != SEGQ_OK) return rc;
+        c.workspace = ptr;
+        c.workspace_bytes = SCRATCH_BYTES;
+    }
+    return gemm_impl(&c, static_cast<hipStream_t>(stream));
 }
 
 int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream) {

@@ -1,0 +1,120 @@
+"""The allocation-free GEMM entry point (segq_gemm_noalloc), through the C ABI.
+
+It must give what segq_gemm gives when the caller lends a workspace of
+segq_gemm_workspace_bytes(d) bytes: bit for bit, since the same kernels make the same
+decisions.  Every case is called twice in a row, the second time on a smaller problem,
+so that what the first call left in the library's scratch array is there when the second
+one runs.  Collected last (file name), so a failure here hides no other test.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import segq_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from segquant_amd import ops as _ops
+    _ops.L.lib()
+    return _ops
+
+
+def _codes(shape, fmt, seed):
+    g = np.random.default_rng(seed)
+    if fmt == O.FMT_INT8:
+        return torch.from_numpy(g.integers(-128, 128, size=shape).astype(np.int8)).to(DEV)
+    if fmt == O.FMT_INT4:
+        return torch.from_numpy(g.integers(0, 256, size=(shape[0], shape[1] // 2)).astype(np.uint8)).to(DEV)
+    c = g.integers(0, 256, size=shape).astype(np.uint8)
+    c[(c & 0x7F) == 0x7F] = 0x3A
+    return torch.from_numpy(c).to(DEV)
+
+
+def _both(ops, make_desc):
+    """(result of segq_gemm with a lent workspace, result of segq_gemm_noalloc, workspace bytes)"""
+    L = ops.L
+    g = make_desc()
+    need = ops.gemm_workspace_bytes(g)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
+    want = ops.gemm_launch(g, ws if need else None).clone()
+    g2 = make_desc()
+    g2[1].fill_(float("nan") if g2[1].dtype.is_floating_point else 0)
+    before = torch.cuda.memory_allocated()
+    rc = L.lib().segq_gemm_noalloc(C.byref(g2[0]), torch.cuda.current_stream().cuda_stream)
+    L.check(rc)
+    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    return want, g2[1], need
+
+
+def _split_case(ops, M, N, K, fmt, seed):
+    a, b = _codes((M, K), fmt, seed), _codes((N, K), fmt, seed + 1)
+    g = torch.Generator().manual_seed(seed)
+    sx = (torch.rand(M, generator=g) + 0.5).to(DEV)
+    sw = (torch.rand(N, generator=g) + 0.5).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    return lambda: ops.gemm_desc(a, b, [ops.Range(0, K, sx, sw, 0, 1, 1)], m=M, n=N, a_fmt=fmt, b_fmt=fmt,
+                                 out_dtype=torch.bfloat16, lda=K, ldb=K, bias=bias)
+
+
+def _park_case(ops, M, N, K0, K1, seed):
+    K = K0 + K1
+    fmt = O.FMT_INT8
+    a, a2, b = _codes((M, K), fmt, seed), _codes((M, K), fmt, seed + 1), _codes((N, K), fmt, seed + 2)
+    g = torch.Generator().manual_seed(seed)
+    s0 = (torch.rand(1, generator=g) + 0.5).to(DEV)
+    sx, sx2 = (torch.rand(M, generator=g) + 0.5).to(DEV), (torch.rand(M, generator=g) + 0.5).to(DEV)
+    sw, bias = (torch.rand(N, generator=g) + 0.5).to(DEV), torch.randn(N, generator=g).to(DEV)
+    rg = [ops.Range(0, K0, s0, sw, 0, 0, 1), ops.Range(K0, K1, sx, sw, 0, 1, 1), ops.Range(K0, K1, sx2, sw, 1, 1, 1)]
+    return lambda: ops.gemm_desc(a, b, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K,
+                                 bias=bias, a_neg=a2)
+
+
+def _int4_case(ops, M, N, K, seed):
+    a, b = _codes((M, K), O.FMT_INT8, seed), _codes((N, K), O.FMT_INT4, seed + 1)
+    return lambda: ops.gemm_desc(a, b, [ops.Range(0, K, None, None)], m=M, n=N, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT4,
+                                 out_dtype="acc", lda=K, ldb=K // 2)
+
+
+def test_noalloc_matches_the_lent_workspace_twice_in_a_row(ops):
+    L = ops.L
+    assert L.lib().segq_init() == 0
+    assert L.lib().segq_noalloc_scratch_bytes() == 64 << 20
+    cases = [
+        # few tiles, long K: the K steps of a tile are shared by several workgroups (fp32 partial results)
+        ("split e4m3", _split_case(ops, 512, 1024, 8192, O.FMT_E4M3, 1), _split_case(ops, 384, 512, 4096, O.FMT_E4M3, 5)),
+        ("split int8", _split_case(ops, 512, 768, 8192, O.FMT_INT8, 11), _split_case(ops, 200, 256, 4096, O.FMT_INT8, 15)),
+        # int8 with three ranges: finished ranges parked as fp32
+        ("park", _park_case(ops, 1536, 1408, 256, 512, 21), _park_case(ops, 1300, 1200, 128, 256, 25)),
+        # int4 weights expanded to int8
+        ("int4", _int4_case(ops, 700, 1536, 1024, 31), _int4_case(ops, 130, 200, 256, 35)),
+    ]
+    for name, first, second in cases:
+        for which, case in (("first", first), ("second, smaller", second)):
+            want, got, need = _both(ops, case)
+            assert need > 0, (name, which, "this case was meant to use a workspace")
+            assert torch.equal(want, got), (name, which)
+
+
+def test_noalloc_refuses_what_does_not_fit_and_runs_what_needs_nothing(ops):
+    L = ops.L
+    # 16 shares of 2048 x 3072 fp32 partial results are 403 MB: more than the array holds
+    a, b = _codes((2048, 16384), O.FMT_E4M3, 41), _codes((3072, 16384), O.FMT_E4M3, 42)
+    one = torch.ones(1, device=DEV)
+    g = ops.gemm_desc(a, b, [ops.Range(0, 16384, one, one, 0, 0, 0)], m=2048, n=3072, a_fmt=O.FMT_E4M3, b_fmt=O.FMT_E4M3,
+                      out_dtype=torch.bfloat16, lda=16384, ldb=16384, split_k=16)
+    assert ops.gemm_workspace_bytes(g) > L.lib().segq_noalloc_scratch_bytes()
+    rc = L.lib().segq_gemm_noalloc(C.byref(g[0]), torch.cuda.current_stream().cuda_stream)
+    assert rc == 1 and b"scratch" in L.lib().segq_last_error()
+    # a plain single-range launch has no use for a workspace and is the same launch as segq_gemm
+    a, b = _codes((300, 512), O.FMT_INT8, 43), _codes((260, 512), O.FMT_INT8, 44)
+    mk = lambda: ops.gemm_desc(a, b, [ops.Range(0, 512, None, None)], m=300, n=260, a_fmt=O.FMT_INT8, b_fmt=O.FMT_INT8,
+                               out_dtype="acc", lda=512, ldb=512)
+    want, got, need = _both(ops, mk)
+    assert need == 0 and torch.equal(want, got)
