@@ -19,18 +19,20 @@ if ROOT not in sys.path:
 
 PEAK_TOPS = {"int8": 5000.0, "fpe4m3": 5000.0}  # dense MFMA, TOP/s
 PEAK_HBM = 8000.0                               # GB/s
-# HBM-side bytes per GEMM launch (fetched + written), from the two rocprofv3 --pmc runs
-# summarised in profiles/gemm_pipe_int8_flux_m4608.md (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB,
-# factors from a 256 MiB copy).  Counters cannot be read from inside this process.
-# the GEMM kernels the tile heuristic picks for each configuration's linears (rocprofv3 traces, profiles/)
-GEMM_KERNELS = {
-    1: "segq::gemm_kernel (int8, general)",
-    2: "segq::gemm_pipe_kernel<128,128> / <256,128, two ranges> (e4m3)",
-    3: "segq::gemm_pipe_kernel<192,288> / <288,192> (int8)",
-    4: "segq::gemm_pipe_kernel<128,128, group factors> (int8 x int4 expanded to int8)",
-    5: "segq::gemm_pipe_kernel<288,192> / <128,128> (int8 with parked ranges, e4m3 rescaled in place)",
-}
-MEASURED_TRAFFIC_BYTES = {3: 343.5e6}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def recorded_traffic(config):
+    """HBM-side bytes per GEMM launch from the last rocprofv3 counter runs of this workload
+    (counters cannot be read from inside this process): profiles/hbm_traffic.json, written by
+    `python -m segquant_amd.profile_counters`.  (bytes or None, where the figure comes from)."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE)).get(str(config))
+    except (OSError, ValueError):
+        rec = None
+    if not rec:
+        return None, "no counter run recorded for this workload"
+    return rec["traffic_bytes_per_launch"], f"profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {rec.get('commit', '?')})"
 
 
 def cpu_baseline(specs, rows, repeats=5):
@@ -94,6 +96,9 @@ def main():
                     help="tokens per linear in the CPU baseline sample (0: the whole workload; a few seconds for config 3)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-e4m3", action="store_true", help="skip the supplementary e4m3 pass over the config-3 shapes")
+    ap.add_argument("--overlap", action="store_true",
+                    help="also time the steps with each linear's quantise kernel on a second stream under the previous linear's "
+                         "GEMM (measured on config 3: 7 %% slower than in sequence, the chip being held by its power limit)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")
     args = ap.parse_args()
@@ -123,10 +128,36 @@ def main():
     n_sets = max(2, -(-(768 << 20) // bytes_per_set))
     sets = [[x.to(dev).clone() for x in inputs] for _ in range(n_sets)]
 
+    biases = [layer.bias_data if layer.bias else None for layer in layers]
+
     def step(i):
         xs = sets[i % n_sets]
         for layer, x in zip(layers, xs):
             layer(x)
+
+    side = torch.cuda.Stream()  # default priority, like the main stream
+
+    def step_overlapped(i):
+        """The same launches with the quantise kernel of linear l + 1 enqueued on a second stream,
+        so that it runs (bound by HBM) under the GEMM of linear l (bound by the matrix cores).
+        The linears of a step are independent, which is what makes this legal here."""
+        xs = sets[i % n_sets]
+        work = [layer.optimizer.fused_launches(x, b, fresh=True) for layer, x, b in zip(layers, xs, biases)]
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)  # buffers the allocator hands out again were last used on the main stream
+        ops.quantize_launch(work[0][0])
+        ready = None
+        for l, (q, g, ws) in enumerate(work):
+            nxt = None
+            if l + 1 < len(work):
+                with torch.cuda.stream(side):
+                    ops.quantize_launch(work[l + 1][0])
+                    nxt = torch.cuda.Event()
+                    nxt.record(side)
+            if ready is not None:
+                main.wait_event(ready)
+            ops.gemm_launch(g, ws)
+            ready = nxt
 
     if args.calib_copy:
         src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
@@ -141,38 +172,88 @@ def main():
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(args.ramp + args.warmup + i)
+    t_host = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     wall = t1 - t0
     total_ops = sum(sp.ops for sp in specs)
     value = total_ops * args.steps / wall / 1e12
-    # A second pass of the same steps with a HIP event pair around every launch gives the
-    # per-kernel durations for the roofline figures.  It is kept out of the timed region:
-    # the twelve event records per step cost ~50 us of a ~500 us step.
+    wall_ov = None
+    if args.overlap:
+        # the same steps with quantise launches overlapped with the previous linear's GEMM
+        for i in range(args.warmup):
+            step_overlapped(i)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for i in range(args.steps):
+            step_overlapped(args.warmup + i)
+        torch.cuda.synchronize()
+        wall_ov = time.perf_counter() - t2
+    # Per-kernel durations for the roofline figures, outside the timed region.  GEMM: the same
+    # steps with a HIP event pair around every launch (the records cost a few microseconds per
+    # launch, little against a GEMM).  Quantise: the kernels are ~10-30 us, so each linear's
+    # quantise launch is instead repeated back to back over the rotating inputs between ONE event
+    # pair; its average includes the gaps between launches and agrees with the kernel trace.
     with ops.record_launches() as log:
         for i in range(args.steps):
             step(args.ramp + args.warmup + args.steps + i)
         torch.cuda.synchronize()
+    q_t = q_bytes = 0.0
+    n_q = 0
+    q_detail = []
+    for li, layer in enumerate(layers):
+        # enough distinct inputs (and outputs) that no launch finds its operands in the 256 MB
+        # last-level cache: the rotation of the timed steps is too short when one kernel runs alone
+        sp = specs[li]
+        per_launch = sp.M * sp.K * (inputs[li].element_size() + 1)
+        copies = [xs[li] for xs in sets]
+        while len(copies) * per_launch < (640 << 20):
+            copies.append(copies[0].clone())
+        qs = [layer.optimizer.fused_launches(x, biases[li], fresh=True)[0] for x in copies]
+        reps = max(1, -(-args.steps // len(qs)))
+        for q in qs:
+            ops.quantize_launch(q)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for q in qs:
+                ops.quantize_launch(q)
+        e1.record()
+        torch.cuda.synchronize()
+        info = qs[0][2]
+        nb = info["rows"] * info["cols"] * (info["x_bytes"] + info["code_bytes"] * info["tensors"]) + (4 * info["rows"] if info["dynamic"] else 0)
+        t = e0.elapsed_time(e1) * 1e-3
+        q_t += t
+        q_bytes += nb * reps * len(qs)
+        n_q += reps * len(qs)
+        q_detail.append({"rows": info["rows"], "cols": info["cols"], "us": round(t / (reps * len(qs)) * 1e6, 2),
+                         "GB/s": round(nb * reps * len(qs) / t / 1e9, 1)})
+        del qs, copies
 
-    g_t = g_ops = g_exec = g_bytes = q_t = q_bytes = 0.0
-    n_g = n_q = 0
+    g_t = g_ops = g_exec = g_bytes = 0.0
+    n_g = 0
     for kind, e0, e1, info in log:
+        if kind != "gemm":
+            continue
         ms = e0.elapsed_time(e1)
-        if kind == "gemm":
-            g_t += ms * 1e-3
-            g_ops += 2.0 * info["m"] * info["n"] * info["k_alg"] * info["batch"]
-            g_exec += 2.0 * info["m"] * info["n"] * info["k_exec"] * info["batch"]
-            g_bytes += info["batch"] * (info["m"] * info["k_alg"] + info["n"] * info["k_alg"] * (0.5 if info["b_fmt"] == "int4" else 1.0)
-                                        + 2.0 * info["m"] * info["n"])
-            n_g += 1
-        else:
-            q_t += ms * 1e-3
-            q_bytes += info["rows"] * info["cols"] * (info["x_bytes"] + info["code_bytes"] * info["tensors"])
-            n_q += 1
+        g_t += ms * 1e-3
+        g_ops += 2.0 * info["m"] * info["n"] * info["k_alg"] * info["batch"]
+        g_exec += 2.0 * info["m"] * info["n"] * info["k_exec"] * info["batch"]
+        g_bytes += info["batch"] * (info["m"] * info["k_alg"] + info["n"] * info["k_alg"] * (0.5 if info["b_fmt"] == "int4" else 1.0)
+                                    + 2.0 * info["m"] * info["n"])
+        n_g += 1
+    # the kernels the library picks for these linears, asked of the library itself
+    kernels = []
+    for layer, x, b in zip(layers, sets[0], biases):
+        q, g, ws = layer.optimizer.fused_launches(x, b)
+        plan = ops.gemm_plan(g, ws)
+        kernels.append(plan["kernel"] + (f" x{plan['splits']} K shares" if plan["splits"] > 1 else "") + (" parked ranges" if plan["parked"] else ""))
     fmt = specs[0].act
     peak = PEAK_TOPS[fmt]
     g_tops = g_ops / g_t / 1e12
     q_gbs = q_bytes / q_t / 1e9
+    traffic, traffic_source = recorded_traffic(args.config)
     out = {
         "metric": "seg-GEMM TOPS + % MFMA peak (FLUX shapes, M=4608); quantize kernel GB/s",
         "value": round(value, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ramp_steps": args.ramp,
@@ -181,15 +262,23 @@ def main():
         "config": {"workload": f"config {args.config}: " + ", ".join(f"{s.name} M{s.M} K{s.K} N{s.N} {s.kernel_type}" for s in specs),
                    "step": "activation quantize + segmented GEMM with fused dequant+bias, per linear",
                    "input_dtype": str(specs[0].x_dtype).replace("torch.", ""), "output_dtype": str(specs[0].x_dtype).replace("torch.", "")},
-        "roofline": {"bound": "mfma", "kernel": GEMM_KERNELS.get(args.config, "segq::gemm_pipe_kernel"), "achieved": round(g_tops, 2), "peak": peak,
-                     "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
+        "roofline": {"bound": "mfma", "kernel": " / ".join(dict.fromkeys(kernels)) + f" ({fmt})", "achieved": round(g_tops, 2), "peak": peak,
+                     "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "launches": n_g, "avg_launch_us": round(g_t / max(n_g, 1) * 1e6, 2),
                      "algorithmic_bytes_per_launch": round(g_bytes / max(n_g, 1)),
-                     "executed_tops": round(g_exec / g_t / 1e12, 2)},
-        "quantize": {"bound": "hbm", "kernel": "segq::quant_*_kernel", "achieved": round(q_gbs, 1), "peak": PEAK_HBM,
-                     "unit": "GB/s", "frac": round(q_gbs / PEAK_HBM, 4), "launches": n_q,
-                     "avg_launch_us": round(q_t / max(n_q, 1) * 1e6, 2)},
+                     "executed_tops": round(g_exec / g_t / 1e12, 2),
+                     # the same launches against the HBM roof (the bound of the small-M shapes)
+                     "hbm_GBps": round(g_bytes / g_t / 1e9, 1), "hbm_frac": round(g_bytes / g_t / 1e9 / PEAK_HBM, 4)},
+        "quantize": {"bound": "hbm", "kernel": "segq::quant_dynamic_row_kernel / quant_dynamic_kernel / quant_static_kernel", "achieved": round(q_gbs, 1),
+                     "peak": PEAK_HBM, "unit": "GB/s", "frac": round(q_gbs / PEAK_HBM, 4), "launches": n_q,
+                     "avg_launch_us": round(q_t / max(n_q, 1) * 1e6, 2), "per_linear": q_detail},
+        # host time to enqueue one linear (descriptor fill + one library call), from the timed region
+        "host_us_per_linear": round((t_host - t0) / (args.steps * len(layers)) * 1e6, 2),
     }
+    if wall_ov is not None:
+        out["overlapped"] = {"value": round(total_ops * args.steps / wall_ov / 1e12, 2), "unit": "TOP/s",
+                             "ms_per_step": round(wall_ov / args.steps * 1e3, 4),
+                             "how": "quantise of linear l+1 on a second stream under the GEMM of linear l (the linears of a step are independent)"}
     if args.config == 3 and not args.no_e4m3:
         # Supplementary: the same three shapes with e4m3 codes on both sides (the metric names
         # int8 and fp8 peaks alike), GEMM launches only, same rotation of operands.
@@ -210,7 +299,11 @@ def main():
         t8 = sum(e0.elapsed_time(e1) for kind, e0, e1, _ in log8 if kind == "gemm") * 1e-3
         n8 = sum(1 for kind, *_ in log8 if kind == "gemm")
         ops8 = sum(2.0 * info["m"] * info["n"] * info["k_alg"] for kind, _, _, info in log8 if kind == "gemm")
-        out["e4m3_same_shapes"] = {"bound": "mfma", "kernel": "segq::gemm_pipe_kernel<192,288> / <288,192> (e4m3)",
+        k8 = []
+        for layer, x in zip(layers8, sets8[0]):
+            q, g, ws = layer.optimizer.fused_launches(x, layer.bias_data if layer.bias else None)
+            k8.append(ops.gemm_plan(g, ws)["kernel"])
+        out["e4m3_same_shapes"] = {"bound": "mfma", "kernel": " / ".join(dict.fromkeys(k8)) + " (fpe4m3)",
                                    "achieved": round(ops8 / t8 / 1e12, 2), "peak": PEAK_TOPS["fpe4m3"], "unit": "TFLOP/s",
                                    "frac": round(ops8 / t8 / 1e12 / PEAK_TOPS["fpe4m3"], 4), "launches": n8,
                                    "avg_launch_us": round(t8 / max(n8, 1) * 1e6, 2)}

@@ -256,6 +256,13 @@ int segq_gemm_tile_count(void);
  * allocates its temporaries itself (segquant/src/real_quant/real_gemm.cu:684-698, :855-865). */
 int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes);
 
+/* What segq_gemm(d) would launch, without launching it: the tile id the library picks (as in
+ * segq_gemm_desc.tile), the number of workgroups that share the K steps of a tile (1: no split)
+ * and whether finished ranges are parked in d's workspace.  Any of the three pointers may be
+ * NULL.  For tools that report which kernel a measurement belongs to; no counterpart in the
+ * reference. */
+int segq_gemm_plan(const segq_gemm_desc* d, int32_t* tile, int32_t* splits, int32_t* parked);
+
 /* ------------------------------------------------------------------------
  * segq_gemm for callers that cannot allocate device memory.
  *

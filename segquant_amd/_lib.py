@@ -63,7 +63,7 @@ class GemmDesc(C.Structure):
 
 EXPORTS = (
     "segq_version", "segq_last_error", "segq_quantize", "segq_quantize_weights_scalar",
-    "segq_quantize_weights_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_linear", "segq_fake_e4m3",
+    "segq_quantize_weights_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3",
     "segq_gemm_noalloc", "segq_noalloc_scratch_bytes", "segq_init",
 )
 
@@ -105,6 +105,8 @@ def lib() -> C.CDLL:
     L.segq_gemm.argtypes = [C.POINTER(GemmDesc), C.c_void_p]
     L.segq_gemm_tile_count.restype = C.c_int
     L.segq_gemm_workspace_bytes.argtypes = [C.POINTER(GemmDesc), C.POINTER(C.c_int64)]
+    L.segq_gemm_plan.argtypes = [C.POINTER(GemmDesc), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    L.segq_gemm_plan.restype = C.c_int
     L.segq_gemm_noalloc.argtypes = [C.POINTER(GemmDesc), C.c_void_p]
     L.segq_gemm_noalloc.restype = C.c_int
     L.segq_noalloc_scratch_bytes.restype = C.c_int64
@@ -112,7 +114,7 @@ def lib() -> C.CDLL:
     L.segq_linear.argtypes = [C.POINTER(QuantDesc), C.POINTER(GemmDesc), C.c_void_p]
     L.segq_fake_e4m3.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
     for name in ("segq_quantize", "segq_quantize_weights_scalar", "segq_quantize_weights_rows", "segq_gemm",
-                 "segq_gemm_workspace_bytes", "segq_linear", "segq_fake_e4m3"):
+                 "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3"):
         getattr(L, name).restype = C.c_int
     _lib = L
     return L

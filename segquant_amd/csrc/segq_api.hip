@@ -161,10 +161,19 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* part, i
     }
 }
 
-// need != nullptr: nothing is launched; *need receives the workspace bytes the launch would use if
-// the caller lent as much as the library can make use of.
-static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, int64_t* need = nullptr) {
-    if (need) *need = 0;
+// What a launch would do, for callers that ask before (or instead of) launching.
+struct GemmPlan {
+    int64_t bytes;  // workspace it would use
+    int tile;       // tile id (1-based, as in segq_gemm_desc.tile)
+    int splits;     // workgroups sharing the K steps of a tile (1: none)
+    int parked;     // finished ranges parked in the workspace
+};
+
+// plan != nullptr: nothing is launched; *plan says what the launch would do if the caller lent
+// as much workspace as the library can make use of (probe) or with d's own workspace (!probe).
+static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = nullptr, bool probe = true) {
+    const bool need = plan != nullptr && probe;
+    if (plan) *plan = GemmPlan{0, 0, 1, 0};
     if (!d) return fail(SEGQ_ERR_ARG, "segq_gemm: null descriptor");
     if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
     if (d->m == 0 || d->n == 0) return SEGQ_OK;
@@ -234,9 +243,17 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, int64_t* need = nu
         // expand b to int8 in the caller's workspace and run the int8 kernels on it
         const int64_t kp = (kmax + 31) & ~(int64_t)31;  // whole 16-byte packed chunks
         if (al(ws, 16) && ws_bytes >= d->batch * d->n * kp && kp / 2 <= d->ldb) {
-            if (need) {
-                *need = d->batch * d->n * kp;
-                return SEGQ_OK;
+            if (plan) {  // the plan of the int8 launch on the expanded weights, plus the expansion's room
+                segq_gemm_desc d8 = *d;
+                d8.b_fmt = SEGQ_CODE_I8;
+                d8.b = ws;
+                d8.ldb = kp;
+                d8.batch_stride_b = d->n * kp;
+                d8.workspace = nullptr;
+                d8.workspace_bytes = 0;
+                const int rc = gemm_impl(&d8, st, plan, false);
+                plan->bytes = d->batch * d->n * kp;
+                return rc;
             }
             const int64_t chunks = kp / 32;
             for (int64_t zb = 0; zb < d->batch; ++zb) {
@@ -387,8 +404,11 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, int64_t* need = nu
     const TileCfg& c = TILE_CFGS[cfg];
     p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);
     p.tiles_n = (int32_t)((d->n + c.bn - 1) / c.bn);
-    if (need) {
-        *need = part_bytes + (park ? (int64_t)splits * p.tiles_m * p.tiles_n * c.bm * c.bn * 4 : 0);
+    if (plan) {
+        plan->bytes = part_bytes + (park ? (int64_t)splits * p.tiles_m * p.tiles_n * c.bm * c.bn * 4 : 0);
+        plan->tile = cfg + 1;
+        plan->splits = splits;
+        plan->parked = park ? 1 : 0;
         return SEGQ_OK;
     }
     p.group_m = 8;
@@ -494,7 +514,19 @@ int segq_gemm_tile_count(void) { return NUM_TILE_CFG; }
 
 int segq_gemm_workspace_bytes(const segq_gemm_desc* d, int64_t* bytes) {
     if (!bytes) return fail(SEGQ_ERR_ARG, "segq_gemm_workspace_bytes: null result pointer");
-    return gemm_impl(d, nullptr, bytes);
+    GemmPlan plan;
+    const int rc = gemm_impl(d, nullptr, &plan);
+    *bytes = plan.bytes;
+    return rc;
+}
+
+int segq_gemm_plan(const segq_gemm_desc* d, int32_t* tile, int32_t* splits, int32_t* parked) {
+    GemmPlan plan;
+    const int rc = gemm_impl(d, nullptr, &plan, false);
+    if (tile) *tile = plan.tile;
+    if (splits) *splits = plan.splits;
+    if (parked) *parked = plan.parked;
+    return rc;
 }
 
 int segq_init(void) {
@@ -506,9 +538,10 @@ int segq_init(void) {
 int64_t segq_noalloc_scratch_bytes(void) { return SCRATCH_BYTES; }
 
 int segq_gemm_noalloc(const segq_gemm_desc* d, segq_stream_t stream) {
-    int64_t need = 0;
-    int rc = gemm_impl(d, nullptr, &need);
+    GemmPlan plan;
+    int rc = gemm_impl(d, nullptr, &plan);
     if (rc != SEGQ_OK) return rc;
+    const int64_t need = plan.bytes;
     if (need > SCRATCH_BYTES)
         return fail(SEGQ_ERR_ARG, "segq_gemm_noalloc: this launch would use %lld bytes of workspace, the library's scratch "
                                   "array holds %lld; use segq_gemm with a workspace of the caller's",

@@ -45,8 +45,18 @@ def _need_cuda(*ts):
             raise RuntimeError("libsegq needs tensors on the GPU")
 
 
-def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(device=None) -> int:
+    """The current torch stream of ``device`` (default: the current device) as a hipStream_t."""
+    if device is None or device.index is None:
+        idx = torch.cuda.current_device()
+    else:
+        idx = device.index
+    if _raw_stream is not None:  # the short way: no Stream object is built
+        return _raw_stream(idx)
+    return torch.cuda.current_stream(idx).cuda_stream
 
 
 # When set to a list, every quantise / GEMM launch is bracketed by events on the
@@ -72,6 +82,12 @@ class record_launches:
         global _launch_log
         _launch_log = self._prev
         return False
+
+
+def recording_launches() -> bool:
+    """Whether a ``record_launches`` block is active (kernels are then launched one per call
+    so that each can be bracketed by its own events)."""
+    return _launch_log is not None
 
 
 def _launch(kind, info, fn):
@@ -103,6 +119,14 @@ def quantize(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional
     """Quantise a 2-D float matrix ``x`` (rows, cols) to codes: :func:`quantize_desc` + one
     ``segq_quantize`` launch.  Returns the code tensor, or ``(Xp, Xn)`` when ``two_tensors``."""
     d, result, info, _keep = quantize_desc(x, fmt, scale, scale_neg, **kw)
+    L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
+    return result
+
+
+def quantize_launch(q):
+    """Enqueue the quantise launch described by ``q`` (the tuple :func:`quantize_desc` returns);
+    returns its code tensor(s)."""
+    d, result, info, _keep = q
     L.check(_launch("quantize", info, lambda: L.lib().segq_quantize(C.byref(d), _stream())))
     return result
 
@@ -202,7 +226,7 @@ def int4_workspace(device, nbytes: int) -> torch.Tensor:
     dev = torch.device(device)
     if dev.index is None:
         dev = torch.device(dev.type, torch.cuda.current_device())
-    key = (dev, torch.cuda.current_stream(dev).cuda_stream)
+    key = (dev, _stream(dev))
     ws = _int4_ws.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
@@ -219,6 +243,25 @@ def gemm_workspace_bytes(g) -> int:
     n = C.c_int64(0)
     L.check(L.lib().segq_gemm_workspace_bytes(C.byref(g[0]), C.byref(n)))
     return n.value
+
+
+# tile ids of the 8-wave kernels (segq_gemm_desc.tile) -> rows x columns of the output tile
+TILE_SHAPES = {1: "256x256", 2: "256x128", 3: "128x128", 4: "64x128", 5: "128x256", 6: "256x256", 7: "256x256", 8: "256x128",
+               11: "256x256", 12: "256x128", 13: "128x256", 14: "128x128", 15: "192x288", 16: "288x192"}
+
+
+def gemm_plan(g, workspace: Optional[torch.Tensor] = None) -> dict:
+    """What the library would launch for ``g`` (lent ``workspace``, if given): its tile id and
+    shape, the number of workgroups sharing a tile's K steps, whether ranges are parked
+    (``segq_gemm_plan``)."""
+    d = g[0]
+    if workspace is not None:
+        d.workspace = workspace.data_ptr(); d.workspace_bytes = workspace.numel() * workspace.element_size()
+    tile, splits, parked = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    L.check(L.lib().segq_gemm_plan(C.byref(d), C.byref(tile), C.byref(splits), C.byref(parked)))
+    family = "gemm_pipe_kernel" if tile.value >= 11 else "gemm_kernel"
+    return dict(tile=tile.value, shape=TILE_SHAPES.get(tile.value, "?"), splits=splits.value, parked=bool(parked.value),
+                kernel=f"segq::{family}<{TILE_SHAPES.get(tile.value, '?').replace('x', ',')}>")
 
 
 def gemm_launch(g, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -260,13 +303,16 @@ def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], **kw) -> tor
     return out
 
 
-def linear(q, g) -> torch.Tensor:
+def linear(q, g, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``segq_linear``: the quantise launch described by ``q`` and the GEMM described by ``g`` (the
-    tuples :func:`quantize_desc` and :func:`gemm_desc` return) in one call of the library.  The GEMM
-    must read the code tensor(s) the quantise step writes, and with dynamic scales the scale
-    tensors it fills."""
+    tuples :func:`quantize_desc` and :func:`gemm_desc` return) in one call of the library, the
+    GEMM lent ``workspace`` if given.  The GEMM must read the code tensor(s) the quantise step
+    writes, and with dynamic scales the scale tensors it fills."""
     qd, _codes, qinfo, _k1 = q
     gd, out, ginfo, _k2 = g
+    if workspace is not None:
+        _need_cuda(workspace)
+        gd.workspace = workspace.data_ptr(); gd.workspace_bytes = workspace.numel() * workspace.element_size()
     L.check(_launch("linear", dict(q=qinfo, g=ginfo), lambda: L.lib().segq_linear(C.byref(qd), C.byref(gd), _stream())))
     return out
 

@@ -258,7 +258,29 @@ class DefaultOptimizer(BaseOptimizer):
         return self._plan
 
     def forward_fused(self, x: torch.Tensor, bias=None, pre_op=None, gate=None, col_div=None, addend=None) -> torch.Tensor:
-        """Final (..., out) result in ``x.dtype``: quantise + segmented GEMM with
+        """Final (..., out) result in ``x.dtype``: the two launches of :meth:`fused_launches`
+        through one call of the library (``segq_linear``), or through two when a
+        ``record_launches`` block is timing the kernels apart."""
+        q, g, ws = self.fused_launches(x, bias, pre_op=pre_op, gate=gate, col_div=col_div, addend=addend)
+        if ops.recording_launches():
+            ops.quantize_launch(q)
+            out = ops.gemm_launch(g, ws)
+        else:
+            out = ops.linear(q, g, ws)
+        return out.view(*x.shape[:-1], out.shape[-1])
+
+    def fused_launches(self, x: torch.Tensor, bias=None, pre_op=None, gate=None, col_div=None, addend=None, fresh=False):
+        """What the fused route enqueues for ``x``, not yet launched: the quantise launch
+        (``ops.quantize_desc``), the GEMM that reads its codes (``ops.gemm_desc``, output
+        (M, out) in ``x.dtype``) and the workspace this layer lends it (or None).  Callers that
+        schedule the two themselves (the quantise step of the next layer under this layer's
+        GEMM, say) use ``ops.quantize_launch`` / ``ops.gemm_launch`` on them.  Calls with a token
+        count seen before reuse the code and scale tensors of the previous call on the same
+        stream (launches on one stream run in order, and the codes only live from the quantise
+        launch to the GEMM that follows it); ``fresh=True`` allocates new ones, for callers that
+        hold several launches of one layer at once.
+
+        Quantise + segmented GEMM with
         de-quantisation and bias fused.  Equivalent to ``forward`` followed by
         the recombination of ``SegmentLinear.forward``, with the partial sums of
         input segments combined in fp32 and rounded once.
@@ -276,6 +298,11 @@ class DefaultOptimizer(BaseOptimizer):
         x2 = x.reshape(-1, K)
         if not x2.is_contiguous():
             x2 = x2.contiguous()
+        plain = pre_op is None and gate is None and col_div is None and addend is None
+        if plain:
+            hit = plan.setdefault("launches", {}).get((x2.shape[0], x.dtype, None if bias is None else bias.data_ptr()))
+            if hit is not None:
+                return self._relaunch(hit, x2, fresh)
         if gate is not None:
             gate = gate.reshape(-1, K)
             if not gate.is_contiguous():
@@ -309,11 +336,11 @@ class DefaultOptimizer(BaseOptimizer):
         # operands stream straight into LDS; the single merged tensor would save a
         # third of the quantise traffic but costs the GEMM ~50 % (sign selection in
         # registers), measured on the 4608 x 15360 x 3072 shape.
-        codes = ops.quantize(x2, plan["fa"], pos, neg, row_stride=1 if per_tok else 0,
-                             kseg_bounds=bounds if S > 1 else None, kseg_stride=kstride, dual=dual,
-                             dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual, pre_op=pre_op, gate=gate,
-                             col_div=col_div)
-        codes, codes_neg = codes if dual else (codes, None)
+        q = ops.quantize_desc(x2, plan["fa"], pos, neg, row_stride=1 if per_tok else 0,
+                              kseg_bounds=bounds if S > 1 else None, kseg_stride=kstride, dual=dual,
+                              dual_kseg_mask=mask, dynamic=dyn, two_tensors=dual, pre_op=pre_op, gate=gate,
+                              col_div=col_div)
+        codes, codes_neg = q[1] if dual else (q[1], None)
         ranges = []
         for s in range(S):
             k0, k1 = bounds[s], bounds[s + 1]
@@ -349,5 +376,64 @@ class DefaultOptimizer(BaseOptimizer):
                 need = plan["ws_need"][M] = ops.gemm_workspace_bytes(g)
             if need:
                 ws = ops.int4_workspace(x.device, need)
-        out = ops.gemm_launch(g, ws)
-        return out.view(*x.shape[:-1], N)
+        if plain:
+            # the same descriptors serve every later call with this token count: only the
+            # addresses of what is allocated per call change (see _relaunch)
+            sx_src = []
+            for s_ in range(S):
+                sx_src.append((0, s_))
+                if dual and self.dual_segments[s_]:
+                    sx_src.append((1, s_))
+            plan["launches"][(M, x.dtype, None if bias is None else bias.data_ptr())] = dict(
+                q=(q[0], q[2]), g=(g[0], g[2]), need=0 if ws is None else need, dyn=dyn, dual=dual, S=S, M=M, N=N, sx_src=sx_src,
+                code_shape=tuple(codes.shape), code_dtype=codes.dtype, out_dtype=x.dtype, static=(pos, neg, bias))
+        return q, g, ws
+
+    def _relaunch(self, hit, x2, fresh=False):
+        """The launches of :meth:`fused_launches` for another input of a token count seen before:
+        the cached descriptors with fresh code, scale and output tensors.  (Filling two
+        descriptors field by field costs ~30 us of host time per call, which is more than the
+        kernels of a small linear take.)"""
+        dev = x2.device
+        out = torch.empty((hit["M"], hit["N"]), dtype=hit["out_dtype"], device=dev)
+        ws = ops.int4_workspace(dev, hit["need"]) if hit["need"] else None
+        stream = None
+        if not fresh:
+            stream = ops._stream(dev)
+            reuse = hit.setdefault("buffers", {}).get(stream)
+            if reuse is not None:  # descriptors, codes and scales of the previous call on this stream
+                qd, gd, result, held = reuse
+                qd.x = x2.data_ptr()
+                gd.out = out.data_ptr()
+                keep = (x2, out, held)
+                return (qd, result, hit["q"][1], keep), (gd, out, hit["g"][1], keep), ws
+        # copies of the descriptors: the caller may hold several launches of this layer at once
+        qd = type(hit["q"][0]).from_buffer_copy(hit["q"][0])
+        gd = type(hit["g"][0]).from_buffer_copy(hit["g"][0])
+        codes = torch.empty(hit["code_shape"], dtype=hit["code_dtype"], device=dev)
+        qd.x = x2.data_ptr()
+        qd.codes = gd.a = codes.data_ptr()
+        gd.out = out.data_ptr()
+        held = [codes, hit["static"]]
+        result = codes
+        if hit["dual"]:
+            codes_neg = torch.empty_like(codes)
+            qd.codes_neg = gd.a_neg = codes_neg.data_ptr()
+            held.append(codes_neg)
+            result = (codes, codes_neg)
+        if hit["dyn"]:
+            S, M = hit["S"], hit["M"]
+            pos = torch.empty((S, M), dtype=torch.float32, device=dev)
+            qd.scale = pos.data_ptr()
+            base = [pos.data_ptr(), 0]
+            held.append(pos)
+            if hit["dual"]:
+                neg = torch.empty_like(pos)
+                qd.scale_neg = base[1] = neg.data_ptr()
+                held.append(neg)
+            for i, (which, s_) in enumerate(hit["sx_src"]):
+                gd.ranges[i].sx = base[which] + 4 * M * s_
+        if stream is not None:
+            hit["buffers"][stream] = (qd, gd, result, held)
+        keep = (x2, out, held)
+        return (qd, result, hit["q"][1], keep), (gd, out, hit["g"][1], keep), ws

@@ -226,3 +226,34 @@ def test_unsupported_kernel_type_warns_and_uses_fake_path(capsys):
                           input_quant_args={"real_quant": True}, weight_quant_args={"real_quant": True}, device=DEV)
     assert "Wint4Aint4" in capsys.readouterr().out
     assert layer.optimizer.real_quant is False
+
+
+@pytest.mark.parametrize("config,M", [(1, 64), (2, 96), (3, 80), (4, 3200), (5, 2100)])
+def test_repeated_forwards_reuse_descriptors_and_buffers(config, M):
+    """The layer keeps its launch descriptors per token count and, on one stream, its code and
+    scale tensors: a third call must give what the first gave, a call on other data what a
+    layer that never saw anything else gives, and outputs handed out earlier must stay intact."""
+    from segquant_amd import workloads as W
+    for spec in W.config_linears(config, M=M)[:2]:
+        layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+        twin, _ = W.build_layer(spec, device=DEV, real_quant=True, x=x)
+        g = torch.Generator().manual_seed(5)
+        xa = x.to(spec.x_dtype).to(DEV)
+        xb = (x * (torch.rand(x.shape[1], generator=g) + 0.5)).to(spec.x_dtype).to(DEV)
+        first = layer(xa)            # builds the descriptors
+        first_copy = first.clone()
+        second = layer(xb)           # cached descriptors, first cached buffers
+        third = layer(xa)            # everything reused
+        other_stream = torch.cuda.Stream()
+        other_stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(other_stream):
+            fourth = layer(xb)       # another stream gets buffers of its own
+        torch.cuda.current_stream().wait_stream(other_stream)
+        assert torch.equal(first, first_copy) and torch.equal(third, first), spec.name
+        assert torch.equal(second, twin(xb)) and torch.equal(fourth, second), spec.name
+        q1, g1, _ = layer.optimizer.fused_launches(xa, layer.bias_data, fresh=True)
+        q2, g2, _ = layer.optimizer.fused_launches(xb, layer.bias_data, fresh=True)
+        assert q1[0] is not q2[0] and g1[1].data_ptr() != g2[1].data_ptr()
+        codes1 = q1[1][0] if isinstance(q1[1], tuple) else q1[1]
+        codes2 = q2[1][0] if isinstance(q2[1], tuple) else q2[1]
+        assert codes1.data_ptr() != codes2.data_ptr()
