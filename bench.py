@@ -96,6 +96,9 @@ def main():
                     help="tokens per linear in the CPU baseline sample (0: the whole workload; a few seconds for config 3)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-e4m3", action="store_true", help="skip the supplementary e4m3 pass over the config-3 shapes")
+    ap.add_argument("--producers", action="store_true",
+                    help="config 5 only: also time every linear fed by its two producers (attention output, MLP output before "
+                         "its GELU) through forward_parts, against torch's GELU + concatenation in front of the ordinary forward")
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with each linear's quantise kernel on a second stream under the previous linear's "
                          "GEMM (measured on config 3: 7 %% slower than in sequence, the chip being held by its power limit)")
@@ -275,6 +278,36 @@ def main():
         # host time to enqueue one linear (descriptor fill + one library call), from the timed region
         "host_us_per_linear": round((t_host - t0) / (args.steps * len(layers)) * 1e6, 2),
     }
+    if args.producers and args.config == 5:
+        import torch.nn.functional as Fn
+        res = []
+        for sp, layer in zip(specs, layers):
+            k0 = sp.chunksizes[0]
+            pre = W.make_input(sp, activated=False).to(sp.x_dtype)
+            n_c = max(2, -(-(768 << 20) // (sp.M * sp.K * 3)))
+            parts = [(pre[:, :k0].to(dev).contiguous(), pre[:, k0:].to(dev).contiguous()) for _ in range(n_c)]
+
+            def torch_front(i):
+                a, m = parts[i % n_c]
+                return layer(torch.cat([a, Fn.gelu(m, approximate="tanh")], dim=1))
+
+            def fused_front(i):
+                a, m = parts[i % n_c]
+                return layer.forward_parts([a, m], pre_ops=[None, "gelu_tanh"])
+
+            t = {}
+            for name, fn in (("torch_gelu_cat_then_linear", torch_front), ("forward_parts", fused_front)):
+                for i in range(5):
+                    fn(i)
+                torch.cuda.synchronize()
+                ta = time.perf_counter()
+                for i in range(args.steps):
+                    fn(i)
+                torch.cuda.synchronize()
+                t[name] = (time.perf_counter() - ta) / args.steps * 1e6
+            res.append({"linear": sp.name, **{k: round(v, 1) for k, v in t.items()}})
+            del parts
+        out["producer_fusion_us"] = res
     if wall_ov is not None:
         out["overlapped"] = {"value": round(total_ops * args.steps / wall_ov / 1e12, 2), "unit": "TOP/s",
                              "ms_per_step": round(wall_ov / args.steps * 1e3, 4),

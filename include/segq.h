@@ -147,6 +147,28 @@ int segq_quantize_weights_rows(const void* weights, int32_t w_dtype, int64_t n, 
                                void* codes, int32_t code_fmt, const float* scale_w_rows,
                                segq_stream_t stream);
 
+/* Weight codes with one scale per (output row, group of `group` input channels):
+ *     codes[r][c] = store(weights[r][c] * scales[(c / group) * n + r])
+ * scales is a contiguous (k / group, n) matrix of multiplicative scales, the layout whose
+ * reciprocals segq_gemm takes as group_dequant.  group: a multiple of 16 that divides k (32 for
+ * int4 codes that the GEMM is to read).  One launch for any number of groups.  The reference has
+ * per-tensor and per-row weight scales only (segquant/src/real_quant/real_gemm.cu:538-638); its
+ * GPTQ calibrator quantises group by group on the host (segquant/calibrator/calibrator.py:262-330). */
+int segq_quantize_weights_groups(const void* weights, int32_t w_dtype, int64_t n, int64_t k, void* codes,
+                                 int32_t code_fmt, const float* scales, int64_t group, segq_stream_t stream);
+
+/* int4 weight codes packed down the columns -> packed along the rows.
+ * colpacked: cols * out / 2 bytes, viewed as (cols, out / 2): byte j of input channel c holds
+ * output rows 2j (low nibble) and 2j + 1 (high nibble) -- what the reference's GPTQ loop emits.
+ * rowpacked: out * cols / 2 bytes, (out, cols / 2): byte m of row r holds input channels 2m (low
+ * nibble) and 2m + 1 (high nibble) -- the layout every int4 consumer reads
+ * (segquant/src/real_quant/quantizer.cuh:37-50).  Replaces
+ * GPTQCalibrator.colpacked1d_to_rowpacked1d (segquant/calibrator/calibrator.py:202-223), which
+ * does it with seven torch operators on full-size temporaries.  out and cols even; the buffers
+ * must not alias. */
+int segq_repack_int4_cols_to_rows(const void* colpacked, void* rowpacked, int64_t out, int64_t cols,
+                                  segq_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Segmented GEMM with fused de-quantisation and bias.
  *

@@ -30,6 +30,9 @@ dequant, bias          closed form
 segment semantics      concatenation / summation invariants
 scale formulas         closed forms incl. the 2^-24 epsilon and 127-vs-128
 fake-quant path        identities against the code path (dequantised codes)
+int4 column repack     element-by-element definition (row r, channel c lives in
+                       nibble r & 1 of byte c * out/2 + r/2) and round trip through
+                       unpack_int4
 =====================  =====================================================
 
 The reference's own tests hold no golden vectors for this path, so the pins
@@ -333,6 +336,26 @@ def smooth_divide(x, s, dtype: str = "fp32") -> np.ndarray:
     this bit for bit."""
     sd = round_to_dtype(_f32(s).reshape(1, -1), dtype)
     return round_to_dtype((_f32(x) / sd).astype(np.float32), dtype)
+
+
+def repack_int4_cols_to_rows(colpacked_1d, out: int, cols: int) -> np.ndarray:
+    """The reference's ``GPTQCalibrator.colpacked1d_to_rowpacked1d``
+    (segquant/calibrator/calibrator.py:202-223), step for step in numpy: the flat input is viewed
+    as (cols, out / 2) and transposed, split into low and high nibbles (output rows 2j and 2j + 1),
+    each (out / 2, cols) nibble plane packed two input channels per byte (even channel low), and the
+    two planes interleaved row by row.  Returns the flat (out * cols / 2,) uint8 array."""
+    assert out % 2 == 0 and cols % 2 == 0, "Output and columns must be even for int4 quantization."
+    q = np.asarray(colpacked_1d, dtype=np.uint8).reshape(cols, out // 2).T
+    low, high = q & 0x0F, (q >> 4) & 0x0F
+
+    def pack(arr):
+        return (arr[:, 0::2] | (arr[:, 1::2] << 4)).astype(np.uint8)
+
+    lp, hp = pack(low), pack(high)
+    res = np.empty((lp.shape[0] * 2, lp.shape[1]), dtype=np.uint8)
+    res[0::2] = lp
+    res[1::2] = hp
+    return res.reshape(-1)
 
 
 def group_amax(w, group: int) -> np.ndarray:

@@ -63,7 +63,7 @@ class GemmDesc(C.Structure):
 
 EXPORTS = (
     "segq_version", "segq_last_error", "segq_quantize", "segq_quantize_weights_scalar",
-    "segq_quantize_weights_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3",
+    "segq_quantize_weights_rows", "segq_quantize_weights_groups", "segq_repack_int4_cols_to_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3",
     "segq_gemm_noalloc", "segq_noalloc_scratch_bytes", "segq_init",
 )
 
@@ -102,6 +102,9 @@ def lib() -> C.CDLL:
                                                C.c_int32, C.c_float, C.c_void_p]
     L.segq_quantize_weights_rows.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p,
                                              C.c_int32, C.c_void_p, C.c_void_p]
+    L.segq_quantize_weights_groups.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_int32,
+                                               C.c_void_p, C.c_int64, C.c_void_p]
+    L.segq_repack_int4_cols_to_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
     L.segq_gemm.argtypes = [C.POINTER(GemmDesc), C.c_void_p]
     L.segq_gemm_tile_count.restype = C.c_int
     L.segq_gemm_workspace_bytes.argtypes = [C.POINTER(GemmDesc), C.POINTER(C.c_int64)]
@@ -114,6 +117,7 @@ def lib() -> C.CDLL:
     L.segq_linear.argtypes = [C.POINTER(QuantDesc), C.POINTER(GemmDesc), C.c_void_p]
     L.segq_fake_e4m3.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
     for name in ("segq_quantize", "segq_quantize_weights_scalar", "segq_quantize_weights_rows", "segq_gemm",
+                 "segq_quantize_weights_groups", "segq_repack_int4_cols_to_rows",
                  "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3"):
         getattr(L, name).restype = C.c_int
     _lib = L

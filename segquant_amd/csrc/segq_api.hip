@@ -47,6 +47,9 @@ int reserve_lds(const void* kern, int bytes, unsigned long long* done) {
 
 int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value);
 int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipStream_t st);
+int quantize_groups_impl(const void* w, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t fmt, const float* scales,
+                         int64_t group, hipStream_t st);
+int repack_i4_impl(const void* colpacked, void* rowpacked, int64_t out, int64_t cols, hipStream_t st);
 
 static bool is_float_dtype(int t) { return t == SEGQ_F32 || t == SEGQ_F16 || t == SEGQ_BF16; }
 static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -506,6 +509,15 @@ int segq_quantize_weights_rows(const void* weights, int32_t w_dtype, int64_t n, 
     q.scale = const_cast<float*>(scale_w_rows);
     q.row_stride = 1;
     return quantize_impl(&q, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int segq_quantize_weights_groups(const void* weights, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t code_fmt,
+                                 const float* scales, int64_t group, segq_stream_t stream) {
+    return quantize_groups_impl(weights, w_dtype, n, k, codes, code_fmt, scales, group, static_cast<hipStream_t>(stream));
+}
+
+int segq_repack_int4_cols_to_rows(const void* colpacked, void* rowpacked, int64_t out, int64_t cols, segq_stream_t stream) {
+    return repack_i4_impl(colpacked, rowpacked, out, cols, static_cast<hipStream_t>(stream));
 }
 
 int segq_gemm(const segq_gemm_desc* d, segq_stream_t stream) { return gemm_impl(d, static_cast<hipStream_t>(stream)); }

@@ -25,6 +25,7 @@ struct QuantParams {
     const void* gate; // with a pre_op: x is multiplied by op(gate) instead of being replaced by op(x)
     int64_t ldg;
     const float* col_div;  // per-column divisors (SmoothQuant's s), applied after the pre_op, or null
+    int32_t group;         // > 0: column segments are runs of this many columns (any number of them), kb unused
     int32_t kb[SEGQ_MAX_KSEG + 1];
 };
 
@@ -187,6 +188,7 @@ __device__ __forceinline__ int64_t row_scale_index(const QuantParams& p, int64_t
 }
 
 __device__ __forceinline__ int kseg_of(const QuantParams& p, int col) {
+    if (p.group > 0) return col / p.group;
     int s = 0;
     for (int i = 1; i < p.n_kseg; ++i) s += (col >= p.kb[i]) ? 1 : 0;
     return s;
@@ -551,7 +553,7 @@ __global__ void __launch_bounds__(256) quant_static_kernel(const QuantParams p) 
     const int col = (int)(run - row * cpr) << 4;
     const int ks = kseg_of(p, col);
     const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
-    const bool dual = p.dual && ((p.dual_mask >> ks) & 1u);
+    const bool dual = p.dual && ((p.dual_mask >> (ks & 31)) & 1u);
     const float s_pos = p.scale ? p.scale[si] : p.scale_imm;
     const float s_neg = dual ? p.scale_neg[si] : s_pos;
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
@@ -704,6 +706,76 @@ int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_b
         case SEGQ_F16: return launch_quant_fmt<SEGQ_F16>(p, st);
         default: return launch_quant_fmt<SEGQ_BF16>(p, st);
     }
+}
+
+// Weight codes with one scale per (row, group of `group` contraction columns): the static kernel
+// with its column segments given by a stride instead of a bounds table.
+int quantize_groups_impl(const void* w, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t fmt, const float* scales,
+                         int64_t group, hipStream_t st) {
+    if (n < 0 || k < 0) return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: negative size");
+    if (n == 0 || k == 0) return SEGQ_OK;
+    if (!w || !codes || !scales) return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: null weights, codes or scales");
+    if (group <= 0 || group % 16 || k % group || group > 0x7fffffff)
+        return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: the group size (%lld) must be a multiple of 16 that divides k (%lld)",
+                    (long long)group, (long long)k);
+    if (w_dtype != SEGQ_F32 && w_dtype != SEGQ_F16 && w_dtype != SEGQ_BF16)
+        return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: w_dtype %d is not a float type", w_dtype);
+    if (fmt != SEGQ_CODE_I8 && fmt != SEGQ_CODE_E4M3 && fmt != SEGQ_CODE_I4)
+        return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: unknown code_fmt %d", fmt);
+    const int64_t esz = w_dtype == SEGQ_F32 ? 4 : 2;
+    if ((k * esz) % 16 || !aligned16(w) || (reinterpret_cast<uintptr_t>(codes) % (fmt == SEGQ_CODE_I4 ? 8 : 16)))
+        return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: weights and codes must be 16-byte aligned");
+    if (n * (k / 16) > (int64_t)0x7fffffff * 256 || k > 0x7fffffff || n > 0x7fffffff)
+        return fail(SEGQ_ERR_ARG, "segq_quantize_weights_groups: matrix too large");
+    QuantParams p{};
+    p.x = w; p.codes = codes; p.scale = const_cast<float*>(scales);
+    p.rows = n; p.cols = k; p.ldx = k; p.ldc = fmt == SEGQ_CODE_I4 ? k / 2 : k;
+    p.seg_rows = n; p.row_stride = 1; p.kseg_stride = n;
+    p.x_dtype = w_dtype; p.fmt = fmt; p.n_kseg = 1; p.group = (int32_t)group;
+    p.kb[0] = 0; p.kb[1] = (int32_t)k;
+    switch (w_dtype) {
+        case SEGQ_F32: return launch_quant_fmt<SEGQ_F32>(p, st);
+        case SEGQ_F16: return launch_quant_fmt<SEGQ_F16>(p, st);
+        default: return launch_quant_fmt<SEGQ_BF16>(p, st);
+    }
+}
+
+// int4 codes packed down the columns (two output rows per byte, the layout the reference's GPTQ
+// loop produces) -> packed along the rows (two input channels per byte, the layout the GEMM reads).
+// A workgroup transposes a patch of 64 input channels x 128 output rows through LDS so that both
+// its reads (along the rows of the source) and its writes (along the rows of the result) are
+// contiguous.
+__global__ void __launch_bounds__(256) repack_i4_kernel(const uint8_t* src, uint8_t* dst, int64_t out, int64_t cols) {
+    __shared__ uint8_t tile[64][65];
+    const int64_t half_out = out >> 1, half_cols = cols >> 1;
+    const int64_t c0 = (int64_t)blockIdx.x * 64, j0 = (int64_t)blockIdx.y * 64;
+    for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+        const int c = idx >> 6, j = idx & 63;
+        uint8_t v = 0;
+        if (c0 + c < cols && j0 + j < half_out) v = src[(c0 + c) * half_out + j0 + j];
+        tile[c][j] = v;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 128 * 32; idx += 256) {
+        const int r = idx >> 5, m = idx & 31;  // output row 2 j0 + r, output byte c0 / 2 + m
+        const int sh = (r & 1) * 4;
+        const uint8_t lo = (tile[2 * m][r >> 1] >> sh) & 0xF, hi = (tile[2 * m + 1][r >> 1] >> sh) & 0xF;
+        const int64_t row = 2 * j0 + r, byte = (c0 >> 1) + m;
+        if (row < out && byte < half_cols) dst[row * half_cols + byte] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+int repack_i4_impl(const void* colpacked, void* rowpacked, int64_t out, int64_t cols, hipStream_t st) {
+    if (out < 0 || cols < 0) return fail(SEGQ_ERR_ARG, "segq_repack_int4: negative size");
+    // the reference asserts both even (segquant/calibrator/calibrator.py:204)
+    if ((out | cols) & 1) return fail(SEGQ_ERR_ARG, "segq_repack_int4: out (%lld) and cols (%lld) must be even", (long long)out, (long long)cols);
+    if (out == 0 || cols == 0) return SEGQ_OK;
+    if (!colpacked || !rowpacked || colpacked == rowpacked) return fail(SEGQ_ERR_ARG, "segq_repack_int4: null or aliased buffers");
+    const int64_t gx = (cols + 63) / 64, gy = (out / 2 + 63) / 64;
+    if (gx > 0x7fffffff || gy > 65535) return fail(SEGQ_ERR_ARG, "segq_repack_int4: matrix too large");
+    hipLaunchKernelGGL(repack_i4_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st, static_cast<const uint8_t*>(colpacked),
+                       static_cast<uint8_t*>(rowpacked), out, cols);
+    return check_launch("segq_repack_int4");
 }
 
 int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipStream_t st) {

@@ -205,6 +205,23 @@ class SegmentLinear(nn.Module):
         return res + self.bias_data if self.bias else res
 
 
+    def forward_parts(self, parts, pre_ops=None):
+        """Forward of an input-segmented layer from the tensors that would have been concatenated
+        into its input (one per segment), each optionally still in front of its producer's
+        activation function (``pre_ops[s]`` in "gelu_tanh" | "gelu" | "silu" | None).  Not in the
+        reference, which runs ``torch.cat([...])`` (and the activation) before the linear
+        (backend/torch/modules/transformer_flux.py:91-101): here every part is quantised
+        straight into its column range of the code tensor, so neither the activated tensor
+        nor the concatenation is written to memory.  The layer must have been calibrated on
+        the concatenated, activated input."""
+        opt = self.optimizer
+        pre_ops = list(pre_ops) if pre_ops is not None else [None] * len(parts)
+        if self.seg_mode == "input" and opt.fused_available() and getattr(opt.weight_calibrators[0], "group_size", None) is None:
+            return opt.forward_parts(parts, self.bias_data if self.bias else None, pre_ops)
+        acted = [p if op is None else self._activated(p, op, None) for p, op in zip(parts, pre_ops)]
+        return self.forward(torch.cat(acted, dim=-1))
+
+
 def create_segment_linear(input_dtype: DType, weight_dtype: DType, opt: Optimum, calib: Calibrate, in_features,
                           out_features, opt_kwargs, calib_kwargs, input_quant_args, weight_quant_args, **kwargs):
     return SegmentLinear(in_features, out_features, input_quant_type=input_dtype.value,

@@ -513,8 +513,8 @@ def quantize_weights_groups(fmt: str, weights: torch.Tensor, scales: torch.Tenso
     ``segq_gemm`` takes as ``group_dequant``.  Returns (n, k) codes, or (n, k / 2) bytes
     for int4.  The reference has no group-wise scales
     (segquant/src/real_quant/real_gemm.cu:538-638 takes a scalar or one scale per row);
-    a group is quantised exactly like a K segment with static per-row scales, so this
-    runs on ``segq_quantize`` in slices of at most SEGQ_MAX_KSEG groups.
+    a group is quantised exactly like a K segment with static per-row scales.  One launch
+    (``segq_quantize_weights_groups``) for any number of groups.
     """
     _need_cuda(weights, scales)
     if weights.dim() != 2 or not weights.is_contiguous():
@@ -526,14 +526,25 @@ def quantize_weights_groups(fmt: str, weights: torch.Tensor, scales: torch.Tenso
     if scales.dtype != torch.float32 or tuple(scales.shape) != (ng, n) or not scales.is_contiguous():
         raise RuntimeError(f"scales must be a contiguous float32 ({ng}, {n}) matrix")
     out = torch.empty((n, k // 2 if fmt == FMT_INT4 else k), dtype=code_dtype(fmt), device=weights.device)
-    step = L.SEGQ_MAX_KSEG
-    for g0 in range(0, ng, step):
-        g1 = min(ng, g0 + step)
-        c0, c1 = g0 * group, g1 * group
-        oc0, oc1 = (c0 // 2, c1 // 2) if fmt == FMT_INT4 else (c0, c1)
-        quantize(weights[:, c0:c1], fmt, scales[g0:], row_stride=1,
-                 kseg_bounds=[i * group for i in range(g1 - g0 + 1)], kseg_stride=n, out=out[:, oc0:oc1])
+    L.check(L.lib().segq_quantize_weights_groups(weights.data_ptr(), _dt(weights.dtype), n, k, out.data_ptr(), _CODE[fmt],
+                                                 scales.data_ptr(), group, _stream()))
     return out
+
+
+def repack_int4_cols_to_rows(colpacked: torch.Tensor, out_features: int, cols: int) -> torch.Tensor:
+    """int4 codes packed down the columns, as the reference's GPTQ loop leaves them (a flat uint8
+    tensor read as (cols, out / 2): two output rows per byte), to the row-packed layout every
+    int4 consumer reads: a flat uint8 tensor of ``out * cols / 2`` bytes, (out, cols / 2), two
+    input channels per byte.  Device counterpart of ``GPTQCalibrator.colpacked1d_to_rowpacked1d``
+    (segquant/calibrator/calibrator.py:202-223)."""
+    _need_cuda(colpacked)
+    if out_features % 2 or cols % 2:
+        raise AssertionError("Output and columns must be even for int4 quantization.")
+    if colpacked.dtype != torch.uint8 or colpacked.numel() != out_features * cols // 2 or not colpacked.is_contiguous():
+        raise RuntimeError("colpacked must be a contiguous uint8 tensor of out * cols / 2 bytes")
+    res = torch.empty(out_features * cols // 2, dtype=torch.uint8, device=colpacked.device)
+    L.check(L.lib().segq_repack_int4_cols_to_rows(colpacked.data_ptr(), res.data_ptr(), out_features, cols, _stream()))
+    return res
 
 
 def fake_e4m3fy(inputs: torch.Tensor) -> torch.Tensor:

@@ -319,14 +319,7 @@ class DefaultOptimizer(BaseOptimizer):
             neg = torch.empty_like(pos) if dual else None
             per_tok = True
         else:
-            if "sx" not in plan:
-                def stack(attr):
-                    vals = []
-                    for c, d in zip(self.input_calibrators, self.dual_segments):
-                        vals.append(_as_f32(getattr(c, attr if d else "scale"), x.device).reshape(-1))
-                    return torch.stack(vals)
-                plan["sx"] = (stack("pos_scale"), stack("neg_scale")) if dual else (stack("scale"), None)
-            pos, neg = plan["sx"]  # (S, 1) per segment or (S, M) per token
+            pos, neg = self._static_sx(plan, x.device)  # (S, 1) per segment or (S, M) per token
             per_tok = pos.shape[-1] > 1
             if per_tok and pos.shape[-1] != M:
                 raise RuntimeError(f"static per-token scales were calibrated for {pos.shape[-1]} tokens, got {M}")
@@ -388,6 +381,82 @@ class DefaultOptimizer(BaseOptimizer):
                 q=(q[0], q[2]), g=(g[0], g[2]), need=0 if ws is None else need, dyn=dyn, dual=dual, S=S, M=M, N=N, sx_src=sx_src,
                 code_shape=tuple(codes.shape), code_dtype=codes.dtype, out_dtype=x.dtype, static=(pos, neg, bias))
         return q, g, ws
+
+    def _static_sx(self, plan, device):
+        """Calibrated activation scales stacked over the input segments: (pos, neg) for DualScale
+        layers (a single-scale segment's one scale stands on both sides), (scale, None) otherwise."""
+        if "sx" not in plan:
+            def stack(attr):
+                vals = []
+                for c, d in zip(self.input_calibrators, self.dual_segments):
+                    vals.append(_as_f32(getattr(c, attr if d else "scale"), device).reshape(-1))
+                return torch.stack(vals)
+            plan["sx"] = (stack("pos_scale"), stack("neg_scale")) if self.dual_scale else (stack("scale"), None)
+        return plan["sx"]
+
+    def forward_parts(self, parts, bias=None, pre_ops=None) -> torch.Tensor:
+        """The fused route for a layer whose input is a concatenation, fed by the producers of the
+        parts instead of by the concatenated tensor: part s (M, chunksizes[s]) is quantised straight
+        into columns [k_s, k_s+1) of the one code tensor the GEMM reads, with the activation
+        function ``pre_ops[s]`` of its producer evaluated inside the quantise kernel.  Neither the
+        activated part nor the concatenation is ever written to memory (the reference builds both
+        with torch operators before the linear, backend/torch/modules/transformer_flux.py:91-101:
+        ``torch.cat([attn_output, self.act_mlp(mlp_hidden_states)], dim=2)`` -> ``proj_out``).
+        One quantise launch per part, then the GEMM of :meth:`fused_launches`."""
+        if self.seg_mode != "input" or len(parts) != self.chunks:
+            raise RuntimeError(f"forward_parts takes one tensor per input segment ({self.chunks} of them)")
+        pre_ops = list(pre_ops) if pre_ops is not None else [None] * len(parts)
+        plan = self._plan or self._build_plan(parts[0].device)
+        if plan.get("group_dequant") is not None:
+            raise NotImplementedError("group-wise weight scales take the concatenated input")
+        K, N = plan["K"], plan["N"]
+        S = self.chunks
+        bounds = plan["bounds"]
+        xs = []
+        for s_, part in enumerate(parts):
+            x2 = part.reshape(-1, part.shape[-1])
+            if x2.shape[1] != bounds[s_ + 1] - bounds[s_]:
+                raise RuntimeError(f"part {s_} has {x2.shape[1]} channels, the segment has {bounds[s_ + 1] - bounds[s_]}")
+            xs.append(x2 if x2.is_contiguous() else x2.contiguous())
+        M = xs[0].shape[0]
+        dev, dt = xs[0].device, xs[0].dtype
+        dyn = bool(self.input_calibrators[0].dynamic)
+        dual = self.dual_scale
+        if dyn:
+            pos = torch.empty((S, M), dtype=torch.float32, device=dev)
+            neg = torch.empty_like(pos) if dual else None
+            per_tok = True
+        else:
+            pos, neg = self._static_sx(plan, dev)
+            per_tok = pos.shape[-1] > 1
+            if per_tok and pos.shape[-1] != M:
+                raise RuntimeError(f"static per-token scales were calibrated for {pos.shape[-1]} tokens, got {M}")
+        fa = plan["fa"]
+        codes = torch.empty((M, K), dtype=ops.code_dtype(fa), device=dev)
+        codes_neg = torch.empty_like(codes) if dual else None
+        ranges = []
+        rs = 1 if per_tok else 0
+        for s_, x2 in enumerate(xs):
+            k0, k1 = bounds[s_], bounds[s_ + 1]
+            d_s = bool(dual and self.dual_segments[s_])
+            ops.quantize(x2, fa, pos[s_], neg[s_] if d_s else None, row_stride=rs, dual=d_s, dynamic=dyn, two_tensors=d_s,
+                         out=codes[:, k0:k1], out_neg=codes_neg[:, k0:k1] if d_s else None, pre_op=pre_ops[s_])
+            ranges.append(ops.Range(k0, k1 - k0, pos[s_], plan["sw"], 0, rs, plan["sw_cs"]))
+            if d_s:
+                ranges.append(ops.Range(k0, k1 - k0, neg[s_], plan["sw"], 1, rs, plan["sw_cs"]))
+        g = ops.gemm_desc(codes, plan["w"], ranges, m=M, n=N, a_fmt=fa, b_fmt=plan["fw"], out_dtype=dt, lda=K,
+                          ldb=K // 2 if plan["fw"] == ops.FMT_INT4 else K, bias=bias, a_neg=codes_neg)
+        int4 = plan["fw"] == ops.FMT_INT4
+        int8_ranges = fa == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1
+        ws = None
+        if (M >= 3072) if int4 else (M >= 2048 or not int8_ranges):
+            need = plan.setdefault("ws_need", {}).get(M)
+            if need is None:
+                need = plan["ws_need"][M] = ops.gemm_workspace_bytes(g)
+            if need:
+                ws = ops.int4_workspace(dev, need)
+        out = ops.gemm_launch(g, ws)
+        return out.view(*parts[0].shape[:-1], N)
 
     def _relaunch(self, hit, x2, fresh=False):
         """The launches of :meth:`fused_launches` for another input of a token count seen before:

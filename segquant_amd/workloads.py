@@ -54,8 +54,10 @@ def _gen(spec: LinearSpec, idx: int) -> torch.Generator:
     return torch.Generator().manual_seed(20250 + 10 * spec.config + spec.tensor_index * 3 + idx)
 
 
-def make_input(spec: LinearSpec, M: Optional[int] = None) -> torch.Tensor:
-    """fp32 (M, K) activation tensor of ``spec`` (optionally only the first M rows' worth)."""
+def make_input(spec: LinearSpec, M: Optional[int] = None, activated: bool = True) -> torch.Tensor:
+    """fp32 (M, K) activation tensor of ``spec`` (optionally only the first M rows' worth).
+    ``activated=False`` leaves out the ``gelu_tanh`` of the segments that have one: what their
+    producer holds before its activation function."""
     M = spec.M if M is None else M
     g = _gen(spec, 0)
     K = spec.K
@@ -68,7 +70,7 @@ def make_input(spec: LinearSpec, M: Optional[int] = None) -> torch.Tensor:
         x[:, chan] = z / chi.sqrt()
     else:
         x[:, chan] *= 30.0 if spec.outlier == "x30" else 20.0
-    if spec.gelu_segments:
+    if spec.gelu_segments and activated:
         bounds = segment_bounds(spec)
         for s in spec.gelu_segments:
             a, b = bounds[s], bounds[s + 1]

@@ -896,3 +896,34 @@ def test_segq_linear_one_call_against_the_oracle(ops, mode, fmt):
         bad = ops.gemm_desc(got_codes_t, wd, [ops.Range(0, K, elsewhere, swd, 0, 1, 0)], **kw)
         with pytest.raises(RuntimeError, match="does not write"):
             ops.linear(q, bad)
+
+
+# ------------------------------------------------------------------ weight-side formats
+@pytest.mark.parametrize("out,cols", [(2, 2), (6, 4), (130, 34), (128, 256), (1280, 5120), (3074, 1026)])
+def test_int4_column_to_row_repack_bit_exact(ops, out, cols):
+    """segq_repack_int4_cols_to_rows against the oracle's restatement of the reference's
+    colpacked1d_to_rowpacked1d, over every byte value and on ragged patches."""
+    g = np.random.default_rng(out * 7 + cols)
+    src = g.integers(0, 256, size=cols * out // 2).astype(np.uint8)
+    src[:256] = np.arange(256, dtype=np.uint8)[:src[:256].size]
+    got = ops.repack_int4_cols_to_rows(torch.from_numpy(src).to(DEV), out, cols).cpu().numpy()
+    assert np.array_equal(got, O.repack_int4_cols_to_rows(src, out, cols))
+    with pytest.raises(AssertionError):
+        ops.repack_int4_cols_to_rows(torch.zeros(3, dtype=torch.uint8, device=DEV), 3, 2)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("dt", ["fp32", "bf16"])
+def test_group_wise_weight_codes_one_launch_any_number_of_groups(ops, fmt, dt):
+    """segq_quantize_weights_groups on 40 groups (more than the eight column segments one
+    activation launch takes) and a group size other than 128, bit-exact against the oracle."""
+    for N, K, G in [(48, 5120, 128), (33, 640, 32), (20, 2048, 256)]:
+        g = torch.Generator().manual_seed(N + K)
+        w = (torch.randn(N, K, generator=g) * 0.05).to(TDT[dt])
+        wn = _np(w).astype(np.float32)
+        lim = {O.FMT_INT8: 127.0, O.FMT_INT4: 7.0, O.FMT_E4M3: 448.0}[fmt]
+        scale = (lim / np.maximum(O.group_amax(wn, G), 2.0 ** -24)).astype(np.float32)  # (N, K / G)
+        sc = torch.from_numpy(np.ascontiguousarray(scale.T)).to(DEV)                     # (K / G, N)
+        codes = ops.quantize_weights_groups(fmt, w.to(DEV), sc, G)
+        want = O.quantize_weights_groups(wn, scale, G, fmt)
+        assert np.array_equal(_codes_np(codes, fmt).view(np.uint8), want.view(np.uint8)), (N, K, G)

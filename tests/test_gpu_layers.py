@@ -257,3 +257,32 @@ def test_repeated_forwards_reuse_descriptors_and_buffers(config, M):
         codes1 = q1[1][0] if isinstance(q1[1], tuple) else q1[1]
         codes2 = q2[1][0] if isinstance(q2[1], tuple) else q2[1]
         assert codes1.data_ptr() != codes2.data_ptr()
+
+
+@pytest.mark.parametrize("fmt", ["int8", "fpe4m3"])
+def test_forward_parts_writes_the_concatenation_as_codes(fmt):
+    """Config 5's proj_out fed by its two producers (attention output, MLP output before its
+    GELU): without activation functions the result is bit for bit what the concatenated tensor
+    gives; with the MLP's GELU(tanh) evaluated in the quantise kernel it agrees to the rounding of
+    the codes (hardware exp2 / reciprocal against torch's tanhf move a code by one step on a few
+    elements)."""
+    from segquant_amd import workloads as W
+    spec = [s for s in W.config_linears(5, M=192) if s.act == fmt][0]
+    layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+    k0 = spec.chunksizes[0]
+    pre = W.make_input(spec, activated=False).to(spec.x_dtype).to(DEV)
+    attn, mlp_pre = pre[:, :k0].contiguous(), pre[:, k0:].contiguous()
+    mlp_act = torch.nn.functional.gelu(mlp_pre, approximate="tanh")
+    want = layer(torch.cat([attn, mlp_act], dim=1))
+    same = layer.forward_parts([attn, mlp_act])
+    assert torch.equal(same, want)
+    fused = layer.forward_parts([attn, mlp_pre], pre_ops=[None, "gelu_tanh"])
+    assert fused.shape == want.shape and fused.dtype == want.dtype
+    w32, f32 = want.float(), fused.float()
+    assert (f32 - w32).abs().max().item() <= 2e-2 * w32.abs().max().item()
+    assert ((f32 - w32).abs() > 2.0 ** -7 * w32.abs().max()).float().mean().item() <= 1e-2
+    # the fake path takes the same call
+    fake, _ = W.build_layer(spec, device=DEV, real_quant=False, x=x)
+    a32, m32 = attn.float(), mlp_pre.float()
+    assert torch.equal(fake.forward_parts([a32, m32], pre_ops=[None, "gelu_tanh"]),
+                       fake(torch.cat([a32, torch.nn.functional.gelu(m32, approximate="tanh")], dim=1)))

@@ -384,3 +384,24 @@ def test_custom_operators_have_shape_only_kernels_for_tracing():
     with pytest.raises(RuntimeError):
         torch.ops.segquant_amd.real_quantized_gemm_scaled(torch.zeros(1, 2, 16), torch.zeros(1, 4, 16, dtype=torch.int8),
                                                           torch.ones(1), torch.ones(1), "int8", "int8")
+
+
+def test_forward_parts_on_the_fake_path_is_the_concatenated_forward():
+    """forward_parts([a, b], pre_ops) on a CPU (fake-quant) layer: the parts are activated and
+    concatenated with torch operators and take the ordinary forward."""
+    import torch
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    g = torch.Generator().manual_seed(3)
+    lin = torch.nn.Linear(96, 40)
+    layer = SegmentLinear(96, 40, bias=True, seg_mode="input", chunks=2, chunksizes=[32, 64],
+                          custom_weight_tensor=lin.weight.data, custom_bias_tensor=lin.bias.data,
+                          input_quant_type="int8", weight_quant_type="int8",
+                          input_quant_args={"dual_scale": [False, True]}, weight_quant_args={}, device="cpu")
+    a, b = torch.randn(7, 32, generator=g), torch.randn(7, 64, generator=g)
+    x = torch.cat([a, torch.nn.functional.silu(b)], dim=1)
+    layer.calibrate(x)
+    layer.finish_calibrate()
+    assert torch.equal(layer.forward_parts([a, b], pre_ops=[None, "silu"]), layer(x))
+    with pytest.raises(Exception):
+        SegmentLinear(96, 40, seg_mode="weight", chunks=2, input_quant_type="int8", weight_quant_type="int8",
+                      device="cpu").optimizer.forward_parts([a, b])

@@ -420,3 +420,27 @@ def test_dequant_dual_against_fp64_closed_form_and_reductions():
     # (c) reductions
     assert np.array_equal(O.dequant_dual(yp2, np.zeros_like(yp2), pos, neg, sw), O.dequant(yp2, pos, sw))
     assert np.array_equal(O.dequant_dual(yp2, yn2, pos, pos, sw), O.dequant(yp2 + yn2, pos, sw))
+
+
+def test_int4_column_to_row_repack_against_its_elementwise_definition():
+    """repack_int4_cols_to_rows (segquant/calibrator/calibrator.py:202-223) pinned by the layouts'
+    definitions, element by element: the source holds value (row r, channel c) in nibble r & 1 of
+    byte c * out/2 + r/2; the result must hold it in nibble c & 1 of byte r * cols/2 + c/2, which
+    is what unpack_int4 reads.  Shapes where out != cols so a transposed view cannot pass."""
+    g = np.random.default_rng(5)
+    for out, cols in [(2, 2), (4, 6), (6, 4), (16, 2), (2, 16), (34, 130), (130, 34)]:
+        vals = g.integers(0, 16, size=(out, cols)).astype(np.uint8)  # nibble of (row, channel)
+        src = np.zeros(cols * out // 2, dtype=np.uint8)
+        for r in range(out):
+            for c in range(cols):
+                src[c * (out // 2) + r // 2] |= vals[r, c] << (4 * (r & 1))
+        got = O.repack_int4_cols_to_rows(src, out, cols)
+        want = np.zeros(out * cols // 2, dtype=np.uint8)
+        for r in range(out):
+            for c in range(cols):
+                want[r * (cols // 2) + c // 2] |= vals[r, c] << (4 * (c & 1))
+        assert np.array_equal(got, want), (out, cols)
+        signed = ((vals.astype(np.int16) ^ 8) - 8).astype(np.int8)  # two's complement nibbles
+        assert np.array_equal(np.stack([O.unpack_int4(row) for row in got.reshape(out, cols // 2)]), signed)
+    with pytest.raises(AssertionError):
+        O.repack_int4_cols_to_rows(np.zeros(3, dtype=np.uint8), 3, 2)
