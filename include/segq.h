@@ -263,6 +263,21 @@ typedef struct segq_gemm_desc {
                          * compute units; no counterpart in the reference (its GemmUniversal runs one K
                          * slice per problem: mode kGemm with batch_count 1,
                          * segquant/src/real_quant/real_gemm.cu:281-285 and :424-445). */
+    const void* lowrank_t;  /* device or NULL.  A low-rank branch added to the result before its one rounding:
+                         *   out[m][n] += sum_{k < lowrank_rank} lowrank_t[m][k] * lowrank_l2t[n][k]
+                         * computed on the matrix cores inside the epilogue (16-bit operands, fp32 sums), so the
+                         * (m, n) product is never written to memory.  This is the inference-time branch of the
+                         * reference's SVD optimiser, x L1 L2 with T = x L1 of shape (m, rank) and L2 of shape
+                         * (rank, n), which there are two bmm launches and an addition of full-size tensors
+                         * (segquant/optimum/optimizer.py:698-731).  Both matrices are in out_dtype, which must
+                         * be F16 or BF16; rows 16-byte aligned.  Needs plain 8-bit codes on both sides, K ranges
+                         * in multiples of 128, batch == 1; not combined with split_k.  Otherwise
+                         * SEGQ_ERR_UNSUPPORTED: pass the product as addend instead. */
+    int64_t ld_lowrank_t;   /* elements; multiple of 8, >= lowrank_rank */
+    const void* lowrank_l2t; /* device: (n, lowrank_rank), i.e. L2 transposed, the contraction index contiguous */
+    int64_t ld_lowrank_l2t;
+    int32_t lowrank_rank;   /* multiple of 32, at most 512; 0 with lowrank_t == NULL */
+    int32_t reserved2;
     segq_krange ranges[SEGQ_MAX_RANGES];
 } segq_gemm_desc;
 

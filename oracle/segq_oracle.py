@@ -30,6 +30,10 @@ dequant, bias          closed form
 segment semantics      concatenation / summation invariants
 scale formulas         closed forms incl. the 2^-24 epsilon and 127-vs-128
 fake-quant path        identities against the code path (dequantised codes)
+smooth / svd split     limits of the formula (alpha 0 and 1, epsilon, clamp); the split
+                       reassembles the weight and its residual has the energy of
+                       the discarded singular values (Eckart-Young); x W^T is
+                       unchanged by smoothing
 int4 column repack     element-by-element definition (row r, channel c lives in
                        nibble r & 1 of byte c * out/2 + r/2) and round trip through
                        unpack_int4
@@ -356,6 +360,46 @@ def repack_int4_cols_to_rows(colpacked_1d, out: int, cols: int) -> np.ndarray:
     res[0::2] = lp
     res[1::2] = hp
     return res.reshape(-1)
+
+
+def smooth_factors(max_x, max_w, alpha: float) -> np.ndarray:
+    """SmoothQuant's per-input-channel factor ``s = max_x^alpha / max_w^(1 - alpha)``; entries at or
+    below 2^-31 become 1; the result is clamped to [1e-4, 1e4], fp32
+    (segquant/optimum/optimizer.py:440-457)."""
+    mx, mw = _f32(max_x), _f32(max_w)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        s = (mx ** np.float32(alpha)) / (mw ** np.float32(1 - alpha))
+    s = np.where(s <= 1.0 / (1 << 31), np.float32(1.0), s).astype(np.float32)
+    return np.clip(s, np.float32(1e-4), np.float32(1e4)).astype(np.float32)
+
+
+def svd_split(w_smooth, rank: int):
+    """The SVD optimiser's split of a smoothed weight chunk (out, in), in fp64
+    (segquant/optimum/optimizer.py:640-684): with ``W^T = U S V^T``, ``L1 = U_r S_r`` (in, r),
+    ``L2 = V_r^T`` (r, out) and the residual ``W - (L1 L2)^T`` (out, in) that gets quantised."""
+    t = np.asarray(w_smooth, dtype=np.float64).T
+    u, sv, vt = np.linalg.svd(t, full_matrices=False)
+    l1 = u[:, :rank] * sv[:rank]
+    l2 = vt[:rank, :]
+    return l1, l2, (t - l1 @ l2).T
+
+
+def smooth_svd_linear(x, s, res_codes, scale_x, scale_w, fmt_a: str, fmt_w: str, l1=None, l2=None, bias=None) -> np.ndarray:
+    """One chunk of a smoothed (and optionally low-rank-split) linear in fp64, as the reference's
+    forward composes it (optimizer.py:514-517, :724-731): the quantised product of ``x / s`` with
+    the residual's codes, de-quantised, plus ``(x / s) L1 L2``.  ``x`` (M, K) fp32 values already
+    in the input's dtype grid, ``s`` (K,), per-tensor or per-row ``scale_x``, per-tensor or
+    per-column ``scale_w``."""
+    xs = _f32(x) / _f32(s)[None, :]
+    sx = np.asarray(scale_x, dtype=np.float32).reshape(-1)
+    codes = quantize_act(xs[None], sx, fmt_a)[0]
+    sw = np.asarray(scale_w, dtype=np.float64).reshape(1, -1)
+    out = gemm_acc(codes, res_codes, fmt_a, fmt_w) / (sx.astype(np.float64).reshape(-1, 1) * sw)
+    if l1 is not None:
+        out = out + (xs.astype(np.float64) @ np.asarray(l1, dtype=np.float64)) @ np.asarray(l2, dtype=np.float64)
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.float64).reshape(1, -1)
+    return out
 
 
 def group_amax(w, group: int) -> np.ndarray:

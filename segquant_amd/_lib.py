@@ -57,6 +57,8 @@ class GemmDesc(C.Structure):
         ("n_ranges", C.c_int32), ("tile", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
         ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64),
         ("addend", C.c_void_p), ("ld_addend", C.c_int64), ("split_k", C.c_int64),
+        ("lowrank_t", C.c_void_p), ("ld_lowrank_t", C.c_int64), ("lowrank_l2t", C.c_void_p), ("ld_lowrank_l2t", C.c_int64),
+        ("lowrank_rank", C.c_int32), ("reserved2", C.c_int32),
         ("ranges", KRange * SEGQ_MAX_RANGES),
     ]
 

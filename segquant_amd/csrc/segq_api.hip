@@ -196,6 +196,18 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     if (d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
     if (d->addend && (d->out_dtype == SEGQ_ACC || d->ld_addend < d->n))
         return fail(SEGQ_ERR_ARG, "segq_gemm: an addend needs a float output and ld_addend >= n");
+    const bool lowrank = d->lowrank_t != nullptr || d->lowrank_rank != 0;
+    if (lowrank) {
+        if (!d->lowrank_t || !d->lowrank_l2t || d->lowrank_rank <= 0 || d->lowrank_rank % 32 || d->lowrank_rank > 512)
+            return fail(SEGQ_ERR_ARG, "segq_gemm: the low-rank branch needs both matrices and a rank that is a multiple of 32, at most 512");
+        if (d->out_dtype != SEGQ_BF16 && d->out_dtype != SEGQ_F16)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: the low-rank branch runs in the output's 16-bit dtype (out_dtype F16 or BF16)");
+        if (d->ld_lowrank_t < d->lowrank_rank || d->ld_lowrank_l2t < d->lowrank_rank || d->ld_lowrank_t % 8 || d->ld_lowrank_l2t % 8 ||
+            !al(d->lowrank_t, 16) || !al(d->lowrank_l2t, 16))
+            return fail(SEGQ_ERR_ARG, "segq_gemm: low-rank matrices need 16-byte aligned rows of at least lowrank_rank elements");
+        if (d->batch != 1 || d->split_k > 1)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: the low-rank branch needs batch == 1 and no split_k");
+    }
     const bool groups = d->group_dequant != nullptr;
     if (groups) {
         if (!(i8 || w4) || d->batch != 1 || d->out_dtype == SEGQ_ACC || d->group_dequant_stride < d->n || !al(d->group_dequant, 4))
@@ -343,7 +355,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     int splits = 1;
     int64_t part_bytes = 0;
     {
-        const bool can = plain8 && wide_ok && d->batch == 1 && !groups && d->out_dtype != SEGQ_ACC && ws && al(ws, 16) &&
+        const bool can = plain8 && wide_ok && d->batch == 1 && !groups && !lowrank && d->out_dtype != SEGQ_ACC && ws && al(ws, 16) &&
                          d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG);
         const int64_t total_steps = ktotal / 128;
         if (d->split_k > 1 && !can)
@@ -403,6 +415,18 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     } else if (cfg >= FIRST_BIG_CFG) {
         if (!wide_ok || w4 || fold)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d needs one range, 8-bit weights and K in multiples of 128", cfg + 1);
+    }
+    if (lowrank) {
+        // small problems, which would otherwise go to the general kernel: the smallest 8-wave tile
+        if (d->tile == 0 && cfg < FIRST_WIDE_CFG && plain8 && wide_ok && splits == 1) cfg = FIRST_WIDE_CFG + 3;
+        if (cfg < FIRST_WIDE_CFG || !plain8 || !wide_ok)
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: the low-rank branch needs plain 8-bit codes on both sides, K ranges in multiples "
+                                              "of 128 and a shape the 8-wave kernels serve; pass the product as addend instead");
+        p.lr_t = static_cast<const uint16_t*>(d->lowrank_t);
+        p.lr_l2 = static_cast<const uint16_t*>(d->lowrank_l2t);
+        p.lr_ldt = d->ld_lowrank_t;
+        p.lr_ldl = d->ld_lowrank_l2t;
+        p.lr_rank = d->lowrank_rank;
     }
     const TileCfg& c = TILE_CFGS[cfg];
     p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);

@@ -55,6 +55,11 @@ struct GemmParams {
     float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
     const float* grw;     // group-wise de-quantisation factors [K / 128][grw_gs], or null
     int64_t grw_gs;
+    const uint16_t* lr_t;   // low-rank branch: T (M x lr_rank) and L2^T (N x lr_rank) in the output's 16-bit dtype, or null
+    const uint16_t* lr_l2;
+    int64_t lr_ldt, lr_ldl;  // their row strides in elements
+    int32_t lr_rank;         // multiple of 32; 0: no low-rank branch
+    int32_t pad3_;
     KRange r[SEGQ_MAX_RANGES];
 };
 

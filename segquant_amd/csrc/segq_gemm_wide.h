@@ -459,6 +459,42 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
     wide_epilogue<BM, BN, WGM, WGN, FMT, B4, FOLD>(p, acc, accf, smem, z, m0, n0, wave, lane);
 }
 
+// Low-rank branch of the epilogue: of[a][b] += sum_k L2T[n][k] T[m][k] over k < lr_rank, on the
+// matrix cores (v_mfma_f32_16x16x32_bf16 / _f16, fp32 accumulation), for the wave's WM x WN
+// patch at (m_row0, n_col0).  `of` holds the de-quantised sums in output units in the lane layout
+// of the accumulators (four consecutive columns of one row per lane and block), which is also
+// the result layout of these MFMAs with L2T as the first operand.  Both fragments are 16 rows of
+// 32 contiguous 16-bit values: a lane reads the 16 bytes of its row at k + 8 lgrp straight from
+// memory (T and L2T are small and stay in the L2).
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+template <int TM, int TN>
+__device__ __forceinline__ void lowrank_accumulate(const GemmParams& p, v4f (&of)[TN][TM], int m_row0, int n_col0, int lane) {
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    const bool bf = p.out_dtype == SEGQ_BF16;
+    for (int kk = 0; kk < p.lr_rank; kk += 32) {
+        uint4 tf[TM];
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int64_t m = min(m_row0 + b * 16 + lrow, p.M - 1);
+            tf[b] = *reinterpret_cast<const uint4*>(p.lr_t + m * p.lr_ldt + kk + lgrp * 8);
+        }
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            const int64_t n = min(n_col0 + a * 16 + lrow, p.N - 1);
+            const uint4 lf = *reinterpret_cast<const uint4*>(p.lr_l2 + n * p.lr_ldl + kk + lgrp * 8);
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                if (bf)
+                    of[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, lf), __builtin_bit_cast(v8bf, tf[b]), of[a][b], 0, 0, 0);
+                else
+                    of[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, lf), __builtin_bit_cast(v8h, tf[b]), of[a][b], 0, 0, 0);
+            }
+        }
+    }
+}
+
 // Software-pipelined variant for plain int8 operands (both straight to LDS) with
 // NS LDS stages.  Two stages are what is instantiated: on FLUX shapes three and
 // four stages measured slower (they cost a co-resident workgroup or buy nothing,
@@ -1025,6 +1061,31 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     if (s < steps) step(std::false_type{}, std::false_type{});
     if constexpr (ACCF) {
         if (dirty) fold(cr);
+    }
+    if (p.lr_rank > 0) {
+        // Low-rank branch (out += T L2): the sums go to output units first (1 / (sx sw) of the range
+        // they are in units of, from the vectors parked in LDS), the low-rank product joins them in
+        // fp32 on the matrix cores, and the epilogue then only adds the bias and rounds once.
+        v4f of[TN][TM];
+        [[maybe_unused]] const bool parked = r_begin < r_last;
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const float rx = ACCF ? 1.0f : epi[wm * WM + b * 16 + lrow];
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                v4f t;
+                if constexpr (HASF) t = accf[a][b];
+                else t = __builtin_convertvector(acc[a][b], v4f);
+                if constexpr (PARK) {
+                    if (parked) t += slot[(a * TM + b) * NT];
+                }
+                if constexpr (!ACCF) t = t * (*reinterpret_cast<const v4f*>(epi + BM + wn * WN + a * 16 + 4 * lgrp) * rx);
+                of[a][b] = t;
+            }
+        }
+        lowrank_accumulate<TM, TN>(p, of, m0 + wm * WM, n0 + wn * WN, lane);
+        wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, true>(p, of, of, smem, z, m0, n0, wave, lane, r_epi, epi);
+        return;
     }
     if constexpr (GRP) {
         v4f none[1][1];

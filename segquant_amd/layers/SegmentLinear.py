@@ -28,6 +28,7 @@ import torch.nn as nn
 from ..calibrator.calibrator import CalibratorRegistry
 from ..config import Calibrate, DType, Optimum
 from ..optimum.optimizer import OptimizerRegistry
+from ..optimum import smooth as _smooth  # noqa: F401  (registers the "smooth" and "svd" optimisers)
 from ..utils.extension import _KERNELS, kernels_available
 from . import ext_dict
 from .segment_tensor_manager import InputSegmentTensorManager, WeightSegmentTensorManager
@@ -106,9 +107,17 @@ class SegmentLinear(nn.Module):
         weight_quant_args["real_quant"] = real_quant
 
         self.opt_type = opt_type
-        if opt_type != "default":
-            raise NotImplementedError(f"optimiser '{opt_type}' is outside the kernel path this package implements")
-        n_w = 1 if seg_mode == "input" else chunks
+        if opt_type not in ("default", "smooth", "svd"):
+            raise ValueError(f"Optimizer '{opt_type}' not found in registry.")
+        # calibrators per optimiser, as the reference lays them out (SegmentLinear.py:118-128): the
+        # default optimiser has one per segment on the segmented side and one on the other, the
+        # smoothing ones a pair per chunk
+        if opt_type == "default":
+            n_w = 1 if seg_mode == "input" else chunks
+        else:
+            n_w = n_in = chunks
+            if len(dual_segments) != chunks:
+                dual_segments = dual_segments * chunks
 
         weight_manager = WeightSegmentTensorManager(weight, seg_mode=seg_mode, segments=chunks,
                                                     segment_size=self.chunksizes[0])
@@ -132,6 +141,14 @@ class SegmentLinear(nn.Module):
         return (f"SegmentLinear(\n  in_features={self.in_features}, out_features={self.out_features}, "
                 f"seg_mode={self.seg_mode},\n  chunks={self.chunks}, chunksize={self.chunksizes},\n"
                 f"  opt={self.optimizer!r}\n)")
+
+    def trace(self, input_data):
+        """Smoothing optimisers only: record the activation maxima of a calibration batch."""
+        self.optimizer.trace(self._manager(input_data))
+
+    def smooth(self):
+        """Smoothing optimisers only: fix the per-channel factors (and the low-rank split)."""
+        self.optimizer.smooth()
 
     def calibrate(self, input_data):
         self.optimizer.calibrate(self._manager(input_data))

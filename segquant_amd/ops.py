@@ -323,9 +323,13 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
          tile: int = 0, workspace: Optional[torch.Tensor] = None,
          group_dequant: Optional[torch.Tensor] = None, split_k: int = 0,
-         addend: Optional[torch.Tensor] = None):
+         addend: Optional[torch.Tensor] = None, lowrank=None):
     """The ``segq_gemm_desc`` of a segmented GEMM with fused de-quantisation and bias, its output
     tensor, the launch's description and the tensors the descriptor points into.
+
+    ``lowrank``: a pair ``(T, L2T)`` of 16-bit matrices in the output's dtype, (m, r) and (n, r)
+    with r a multiple of 32: ``T @ L2T.T`` is added to the result inside the epilogue (the SVD
+    optimiser's branch x L1 L2 with T = x L1; see ``segq_gemm_desc.lowrank_t``).
 
     ``out_dtype`` is a torch float dtype, or the string ``"acc"`` for the raw
     accumulators (int32 for integer codes, float32 for e4m3).  ``workspace``: a
@@ -364,6 +368,15 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
         if raw or addend.dtype != tdt or addend.shape != out.shape or not addend.is_contiguous():
             raise RuntimeError("addend must be a contiguous tensor of the output's shape and dtype")
         d.addend = addend.data_ptr(); d.ld_addend = n
+    if lowrank is not None:
+        t_lr, l2t = lowrank
+        _need_cuda(t_lr, l2t)
+        if raw or t_lr.dtype != tdt or l2t.dtype != tdt or t_lr.dim() != 2 or l2t.dim() != 2 or t_lr.shape[0] != m or \
+                l2t.shape[0] != n or t_lr.shape[1] != l2t.shape[1] or t_lr.stride(1) != 1 or l2t.stride(1) != 1:
+            raise RuntimeError("lowrank is (T (m, r), L2T (n, r)) in the output's dtype with contiguous rows")
+        d.lowrank_t = t_lr.data_ptr(); d.ld_lowrank_t = t_lr.stride(0)
+        d.lowrank_l2t = l2t.data_ptr(); d.ld_lowrank_l2t = l2t.stride(0)
+        d.lowrank_rank = t_lr.shape[1]
     if group_dequant is not None:
         _need_cuda(group_dequant)
         if group_dequant.dtype != torch.float32 or group_dequant.dim() != 2 or group_dequant.stride(1) != 1:
@@ -381,7 +394,7 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
         kr.sw = r.sw.data_ptr() if r.sw is not None else None
     info = dict(m=m, n=n, batch=batch, k_alg=sum(r.k_len for r in ranges if r.a_sel in (0, 2)),
                 k_exec=sum(r.k_len for r in ranges), a_fmt=a_fmt, b_fmt=b_fmt)
-    return d, out, info, (a, b, a_neg, bias, workspace, group_dequant, addend, out, list(ranges))
+    return d, out, info, (a, b, a_neg, bias, workspace, group_dequant, addend, lowrank, out, list(ranges))
 
 
 # ---------------------------------------------------------------------------

@@ -298,7 +298,9 @@ class DefaultOptimizer(BaseOptimizer):
         x2 = x.reshape(-1, K)
         if not x2.is_contiguous():
             x2 = x2.contiguous()
-        plain = pre_op is None and gate is None and col_div is None and addend is None
+        if col_div is None:
+            col_div = plan.get("col_div")  # a smoothed layer's own divisors
+        plain = pre_op is None and gate is None and col_div is None and addend is None and "l2t" not in plan
         if plain:
             hit = plan.setdefault("launches", {}).get((x2.shape[0], x.dtype, None if bias is None else bias.data_ptr()))
             if hit is not None:
@@ -338,16 +340,34 @@ class DefaultOptimizer(BaseOptimizer):
         for s in range(S):
             k0, k1 = bounds[s], bounds[s + 1]
             rs = 1 if per_tok else 0
+            sw_s = plan["sw_list"][s] if "sw_list" in plan else plan["sw"]  # smoothed layers: one weight scale per K segment
+            ranges.append(ops.Range(k0, k1 - k0, pos[s], sw_s, 0, rs, plan["sw_cs"]))
             if dual and self.dual_segments[s]:
-                ranges.append(ops.Range(k0, k1 - k0, pos[s], plan["sw"], 0, rs, plan["sw_cs"]))
-                ranges.append(ops.Range(k0, k1 - k0, neg[s], plan["sw"], 1, rs, plan["sw_cs"]))
-            else:
-                ranges.append(ops.Range(k0, k1 - k0, pos[s], plan["sw"], 0, rs, plan["sw_cs"]))
+                ranges.append(ops.Range(k0, k1 - k0, neg[s], sw_s, 1, rs, plan["sw_cs"]))
         ldb = K // 2 if plan["fw"] == ops.FMT_INT4 else K
         gdq = plan.get("group_dequant")
-        g = ops.gemm_desc(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype,
-                          lda=K, ldb=ldb, bias=bias, a_neg=codes_neg, group_dequant=gdq,
-                          addend=None if addend is None else addend.reshape(M, N).contiguous())
+        add2 = None if addend is None else addend.reshape(M, N).contiguous()
+        kw = dict(m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype, lda=K, ldb=ldb, bias=bias, a_neg=codes_neg,
+                  group_dequant=gdq)
+        g = None
+        if "l2t" in plan:
+            # the SVD optimiser's low-rank branch: inside the GEMM's epilogue where the library has a
+            # kernel for it (16-bit dtypes, the 8-wave kernels), as a materialised (M, N) addend otherwise
+            t_lr, l2t = self._lowrank_operands(plan, x2)
+            ok = plan.setdefault("lr_ok", {}).get((M, x.dtype))
+            if ok is None or ok:
+                try:
+                    g = ops.gemm_desc(codes, plan["w"], ranges, addend=add2, lowrank=(t_lr, l2t), **kw)
+                    if ok is None:
+                        ops.gemm_plan(g)
+                except RuntimeError:
+                    g = None
+                plan["lr_ok"][(M, x.dtype)] = g is not None
+            if g is None:
+                low = t_lr @ l2t.t()
+                add2 = low if add2 is None else add2 + low
+        if g is None:
+            g = ops.gemm_desc(codes, plan["w"], ranges, addend=add2, **kw)
         # Whether to lend the library a workspace is this layer's call; how much it could use is
         # the library's (segq_gemm_workspace_bytes), asked once per token count.
         #  * int4 weights and many tokens: the GEMM is bound by the matrix cores, so the weights are

@@ -2,7 +2,7 @@
 calibrated ``SegmentLinear`` modules.
 
 Counterpart of segquant/torch/quantization.py:259-425 for the kernel path:
-default optimiser, amax calibration.  The reference finds segmentation and
+default, smooth and svd optimisers (fixed alpha), amax calibration.  The reference finds segmentation and
 DualScale candidates with a torch.fx pattern detector; graph analysis is
 outside this build, so both are passed in: ``seg_configs`` maps a linear's name
 to ``{"seg_mode", "chunks" | "chunksizes"}`` and ``dual_scale_linears`` names the
@@ -83,6 +83,24 @@ def _run_model(model, loader, device):
             model(*inp) if isinstance(inp, tuple) else model(**inp)
 
 
+def _trace_and_smooth(model, to_smooth, loader, origin_device, target_device):
+    """The two extra passes of the smoothing optimisers (reference quantization.py:110-145, :386-412):
+    run the calibration data once to record activation maxima, then fix the per-channel factors."""
+    hooks = []
+    for name, mod in model.named_modules():
+        if isinstance(mod, nn.Linear) and name in to_smooth:
+            def hook(_m, inp, _out, n=name):
+                to_smooth[n].trace(_move_to_device(inp[0], target_device))
+            hooks.append(mod.register_forward_hook(hook))
+    try:
+        _run_model(model, loader, origin_device)
+    finally:
+        for h in hooks:
+            h.remove()
+    for lin in to_smooth.values():
+        lin.smooth()
+
+
 def _calib_linears(model, new_linears, loader, origin_device, target_device):
     hooks = []
     for name, mod in model.named_modules():
@@ -139,6 +157,11 @@ def quantize(model: nn.Module, calib_data_loader, config=None, tmp_device=None, 
         if name in seg_configs and _config_for(name, final_config).get("seglinear", True):
             seg = seg_configs[name]
         new_linears[name] = _create_linear(lin, name, seg, final_config, dual_scale=name in dual, device=target_device)
+    to_smooth = {k: v for k, v in new_linears.items() if v.opt_type in ("smooth", "svd")}
+    if to_smooth:
+        if verbose:
+            print("start trace and smooth ...")
+        _trace_and_smooth(model, to_smooth, calib_data_loader, origin_device, target_device)
     if verbose:
         print("start calibrate ...")
     _calib_linears(model, new_linears, calib_data_loader, origin_device, target_device)

@@ -102,3 +102,42 @@ def oracle_layer_output(layer, spec, x_np, out_dtype=None, rows=None, cols=None)
     if layer.bias:
         y += _np32(layer.bias_data).astype(np.float64)[csel]
     return y
+
+
+def oracle_smooth_layer_output(layer, fmt_a, fmt_w, x_np, rows=None, cols=None):
+    """Closed form (fp64) of a calibrated smooth / svd SegmentLinear with input segmentation or a
+    single chunk, from the layer's own factors, codes and scales: per K segment i,
+    codes(x_i / s_i) W_i^T / (sx_i sw_i) + (x_i / s_i) L1_i L2_i, plus the bias
+    (segquant/optimum/optimizer.py:514-517, :724-731).  The division is carried out in the
+    input's dtype grid when ``x_np`` holds bf16 / fp16 values (``dtype`` of the layer's input)."""
+    opt = layer.optimizer
+    wq = _unpacked_weight_codes(layer, fmt_w)
+    if rows is not None:
+        x_np = x_np[np.asarray(rows)]
+    csel = np.arange(wq.shape[0]) if cols is None else np.asarray(cols)
+    wq = wq[csel]
+    N, K = wq.shape
+    S = opt.chunks if opt.seg_mode == "input" else 1
+    ksz = K // S
+    y = np.zeros((x_np.shape[0], N))
+    lim = {O.FMT_INT8: 127.0, O.FMT_E4M3: 448.0}[fmt_a]
+    for i in range(S):
+        ks = slice(i * ksz, (i + 1) * ksz)
+        s = _np32(opt.s[i]).astype(np.float32)
+        xs = O.smooth_divide(x_np[:, ks], s, layer._oracle_dtype)
+        cal = opt.input_calibrators[i]
+        if cal.dynamic:
+            sx = O.row_scale_div(np.abs(xs).max(axis=-1), lim)
+        else:
+            sx = np.float32(_np32(torch.as_tensor(cal.scale))).reshape(-1)
+        sw = np.float32(_np32(torch.as_tensor(opt.weight_calibrators[i].scale))).reshape(-1)
+        sw = (np.broadcast_to(sw, (layer.out_features,)) if sw.size == 1 else sw)[csel].astype(np.float64)
+        codes = O.quantize_act(xs[None], sx if sx.size > 1 else sx[:1], fmt_a)[0]
+        y += O.gemm_acc(codes, wq[:, ks], fmt_a, fmt_w) / (sx.astype(np.float64).reshape(-1, 1) * sw[None, :])
+        if getattr(opt, "l1s", None) is not None:
+            l1 = _np32(opt.l1s[i]).astype(np.float64)
+            l2 = _np32(opt.l2s[i]).astype(np.float64)[:, csel]
+            y += (xs.astype(np.float64) @ l1) @ l2
+    if layer.bias:
+        y += _np32(layer.bias_data).astype(np.float64)[csel]
+    return y

@@ -275,3 +275,29 @@ def test_full_size_layers_against_the_oracle(config, M, dtype):
             assert (err <= bound).all(), (spec.name, float((err / bound).max()))
         del layer
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("rank", [32, 64])
+def test_full_size_svd_layer_low_rank_in_the_epilogue(rank):
+    """Configuration 3's mlp_up (4608 x 3072 -> 12288, int8, per-token dynamic activations,
+    per-channel weights, bf16) as an svd layer: SmoothQuant division in the quantise kernel, the
+    rank-r branch added by the GEMM's epilogue.  Row and column bands against the oracle's closed
+    form built from the layer's own factors, codes and scales (optimizer.py:514-517, :724-731)."""
+    from _layer_oracle import _np32, oracle_smooth_layer_output
+    from test_gpu_layers import _smooth_layer
+    M, K, N = 4608, 3072, 12288
+    layer, xd, _ = _smooth_layer("svd", "int8", "weight", 1, M, K, N, torch.bfloat16, True, axis=True, rank=rank, seed=9)
+    assert layer.optimizer.fused_available()
+    out = layer(xd)
+    plan = layer.optimizer._plan
+    assert plan["lr_ok"][(M, torch.bfloat16)] is True  # the epilogue branch ran, not the materialised addend
+    got = _np32(out).astype(np.float64)
+    x_np = _np32(xd)
+    rows, cols = _bands(M, N)
+    for ri, ci in ((rows, None), (None, cols)):
+        want = oracle_smooth_layer_output(layer, "int8", "int8", x_np, rows=ri, cols=ci)
+        sub = got[np.ix_(np.arange(M) if ri is None else ri, np.arange(N) if ci is None else ci)]
+        # T = x (L1 / s), L1 / s and L2 are rounded to bf16 for the matrix cores: 2^-9 each, against the
+        # size of the low-rank term (here of the order of the output itself)
+        assert np.abs(sub - want).max() <= 1.2e-2 * np.abs(want).max()
+        assert np.sqrt(((sub - want) ** 2).mean()) <= 2.5e-3 * np.abs(want).max()

@@ -927,3 +927,66 @@ def test_group_wise_weight_codes_one_launch_any_number_of_groups(ops, fmt, dt):
         codes = ops.quantize_weights_groups(fmt, w.to(DEV), sc, G)
         want = O.quantize_weights_groups(wn, scale, G, fmt)
         assert np.array_equal(_codes_np(codes, fmt).view(np.uint8), want.view(np.uint8)), (N, K, G)
+
+
+# ------------------------------------------------------------------ low-rank branch in the epilogue
+def _e4m3_codes(g, shape):
+    """Moderate e4m3 codes (|value| <= 16) without the NaN patterns."""
+    c = g.integers(0, 256, size=shape).astype(np.uint8)
+    c = (c & 0x80) | np.minimum(c & 0x7F, 0x58)
+    return c.astype(np.uint8)
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("ranges", [1, 3])
+@pytest.mark.parametrize("lend", [False, True])
+def test_gemm_low_rank_branch_in_the_epilogue(ops, fmt, dt, ranges, lend):
+    """out = sum_r A_r B_r^T / (sx_r sw_r) + bias + T L2 with the low-rank product computed by the
+    epilogue's MFMAs: against the fp64 closed form on every 8-wave tile, with one range and with
+    three (a second accumulator set, parked ranges when a workspace is lent, fp32 sums rescaled in
+    place for e4m3), ragged M and N, ranks 32 and 96."""
+    M, N, K = 330, 424, 768
+    g = np.random.default_rng(77)
+    a = g.integers(-128, 128, size=(M, K)).astype(np.int8) if fmt == O.FMT_INT8 else _e4m3_codes(g, (M, K))
+    a2 = g.integers(-128, 128, size=(M, K)).astype(np.int8) if fmt == O.FMT_INT8 else _e4m3_codes(g, (M, K))
+    b = g.integers(-128, 128, size=(N, K)).astype(np.int8) if fmt == O.FMT_INT8 else _e4m3_codes(g, (N, K))
+    av, a2v, bv = (O.code_values(t, fmt) for t in (a, a2, b))
+    tg = torch.Generator().manual_seed(78)
+    sx0 = torch.rand(1, generator=tg) * 50 + 20
+    sx1, sx2 = torch.rand(M, generator=tg) * 50 + 20, torch.rand(M, generator=tg) * 50 + 20
+    sw = torch.rand(N, generator=tg) * 50 + 20
+    bias = torch.randn(N, generator=tg)
+    ad, a2d, bd = (torch.from_numpy(t).to(DEV) for t in (a, a2, b))
+    if ranges == 1:
+        rg = [ops.Range(0, K, sx1.to(DEV), sw.to(DEV), 0, 1, 1)]
+        base = (av @ bv.T) / (sx1.numpy().astype(np.float64)[:, None] * sw.numpy().astype(np.float64)[None, :])
+    else:
+        K0 = 256
+        swd = sw.to(DEV)
+        rg = [ops.Range(0, K0, sx0.to(DEV), swd, 0, 0, 1), ops.Range(K0, K - K0, sx1.to(DEV), swd, 0, 1, 1),
+              ops.Range(K0, K - K0, sx2.to(DEV), swd, 1, 1, 1)]
+        s0, s1, s2, swn = (t.numpy().astype(np.float64) for t in (sx0, sx1, sx2, sw))
+        base = ((av[:, :K0] @ bv[:, :K0].T) / (s0[0] * swn[None, :]) + (av[:, K0:] @ bv[:, K0:].T) / (s1[:, None] * swn[None, :])
+                + (a2v[:, K0:] @ bv[:, K0:].T) / (s2[:, None] * swn[None, :]))
+    for rank in (32, 96):
+        t_lr = (torch.randn(M, rank, generator=tg) * 0.5).to(TDT[dt])
+        l2t = (torch.randn(N, rank, generator=tg) * 0.5).to(TDT[dt])
+        want = base + bias.numpy().astype(np.float64) + t_lr.double().numpy() @ l2t.double().numpy().T
+        ws = torch.empty(ops.park_bytes(M, N), dtype=torch.uint8, device=DEV) if lend else None
+        for tile in (0, 11, 12, 13, 14, 15, 16):
+            if ranges == 3 and fmt == O.FMT_INT8 and not lend and tile in (11, 15, 16):
+                continue  # these tiles have no second accumulator set: they need the workspace
+            out = ops.gemm(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=K, bias=bias.to(DEV),
+                           a_neg=a2d if ranges == 3 else None, tile=tile, workspace=ws, lowrank=(t_lr.to(DEV), l2t.to(DEV)))
+            got = out.float().cpu().numpy().astype(np.float64)
+            ulp = 2.0 ** -8 if dt == "bf16" else 2.0 ** -11
+            tol = ulp * np.abs(want) + (3e-4 if fmt == O.FMT_E4M3 else 1e-5) * np.abs(want).max()
+            assert (np.abs(got - want) <= tol).all(), (tile, rank, float((np.abs(got - want) / tol).max()))
+    # what the branch does not serve is refused, not ignored
+    t_lr, l2t = torch.zeros(M, 32, device=DEV), torch.zeros(N, 32, device=DEV)
+    with pytest.raises(RuntimeError):
+        ops.gemm(ad, bd, rg[:1], m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, lowrank=(t_lr, l2t))
+    with pytest.raises(RuntimeError, match="low-rank"):
+        ops.gemm(ad, bd, rg[:1], m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=K, tile=3,
+                 lowrank=(t_lr.to(TDT[dt]), l2t.to(TDT[dt])))

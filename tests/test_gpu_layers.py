@@ -286,3 +286,69 @@ def test_forward_parts_writes_the_concatenation_as_codes(fmt):
     a32, m32 = attn.float(), mlp_pre.float()
     assert torch.equal(fake.forward_parts([a32, m32], pre_ops=[None, "gelu_tanh"]),
                        fake(torch.cat([a32, torch.nn.functional.gelu(m32, approximate="tanh")], dim=1)))
+
+
+def _smooth_layer(opt_type, fmt, seg_mode, chunks, M, K, N, dtype, dynamic, axis, rank=32, seed=3):
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(N, K, generator=g) * 0.02
+    b = torch.randn(N, generator=g) * 0.01
+    x = torch.randn(M, K, generator=g) * (torch.rand(K, generator=g) * 3 + 0.3)
+    x[:, torch.randperm(K, generator=g)[:max(1, K // 100)]] *= 20.0
+    layer = SegmentLinear(K, N, bias=True, seg_mode=seg_mode, chunks=chunks, custom_weight_tensor=w, custom_bias_tensor=b,
+                          input_quant_type=fmt, weight_quant_type=fmt,
+                          input_quant_args={"real_quant": True, "axis": -1 if (dynamic or axis) else None, "dynamic": dynamic},
+                          weight_quant_args={"real_quant": True, "axis": 1 if axis else None}, opt_type=opt_type,
+                          opt_kwargs={"alpha": 0.5, **({"low_rank": rank, "precision": "float32"} if opt_type == "svd" else {})},
+                          device=DEV)
+    xd = x.to(dtype).to(DEV)
+    layer.trace(xd)
+    layer.smooth()
+    layer.calibrate(xd)
+    layer.finish_calibrate()
+    layer._oracle_dtype = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}[dtype]
+    return layer, xd, (w, b, x)
+
+
+@pytest.mark.parametrize("opt_type", ["smooth", "svd"])
+@pytest.mark.parametrize("fmt", ["int8", "fpe4m3"])
+@pytest.mark.parametrize("seg_mode,chunks", [("weight", 1), ("input", 2)])
+@pytest.mark.parametrize("dtype,dynamic", [(torch.bfloat16, True), (torch.float16, False), (torch.float32, False)])
+def test_smooth_and_svd_layers_fused_route_against_the_oracle(opt_type, fmt, seg_mode, chunks, dtype, dynamic):
+    """Smoothed (and low-rank-split) layers through the fused route: the division by s in the
+    quantise kernel, one range per K segment with its own activation and weight scales, and the
+    low-rank product added by the GEMM's epilogue (16-bit inputs) or as an addend (fp32).
+    Against the oracle's closed form from the layer's own factors; and the reference's route
+    (chunked operator + two batched products) must agree with the fused one."""
+    from _layer_oracle import oracle_smooth_layer_output
+    M, K, N = 200, 512, 384
+    layer, xd, (w, b, x) = _smooth_layer(opt_type, fmt, seg_mode, chunks, M, K, N, dtype, dynamic, axis=True)
+    assert layer.optimizer.fused_available()
+    out = layer(xd)
+    assert out.shape == (M, N) and out.dtype == dtype
+    got = _np32(out).astype(np.float64)
+    want = oracle_smooth_layer_output(layer, fmt, fmt, _np32(xd))
+    scale = np.abs(want).max()
+    # bf16 / fp16: T = x (L1 / s) and L2 are rounded to the input's dtype for the matrix cores
+    tol = {torch.float32: 2e-5, torch.bfloat16: 1.2e-2, torch.float16: 2e-3}[dtype] + (1e-3 if fmt == "fpe4m3" else 0.0)
+    assert np.abs(got - want).max() <= tol * scale, float(np.abs(got - want).max() / scale)
+    chunked = layer(xd, chunked=True)
+    rec = (chunked.sum(0) if seg_mode == "input" else chunked.movedim(0, -2).reshape(M, -1)) + layer.bias_data
+    # (the reference's route computes dynamic scales with torch in the input's dtype, so its codes
+    # differ from the fused route's by a step here and there: compare the two as a whole)
+    assert ((rec.float() - out.float()).norm() / out.float().norm()).item() <= (3e-2 if fmt == "fpe4m3" else 1e-2)
+    # the smoothed, split layer is still the linear it replaces (quantisation error only)
+    ref = torch.nn.functional.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert ((out.float() - ref).norm() / ref.norm()).item() < 0.05
+
+
+def test_smooth_layer_with_output_segments_takes_the_reference_route():
+    """With output segmentation every segment smooths the whole input with its own s, so the layer
+    runs the reference's route: S smoothed, quantised copies of the input through the batched
+    operator.  Checked against the float linear."""
+    M, K, N = 96, 256, 384
+    layer, xd, (w, b, x) = _smooth_layer("svd", "int8", "weight", 3, M, K, N, torch.float32, False, axis=True, rank=16)
+    assert not layer.optimizer.fused_available() and layer.optimizer.real_quant
+    out = layer(xd)
+    ref = torch.nn.functional.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert out.shape == (M, N) and ((out - ref).norm() / ref.norm()).item() < 0.05

@@ -268,8 +268,10 @@ def test_constructor_checks_mirror_the_reference():
     with pytest.raises(ValueError):
         SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8",
                       weight_quant_args={"dual_scale": True}, device="cpu")
-    with pytest.raises(NotImplementedError):
-        SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8", opt_type="smooth", device="cpu")
+    with pytest.raises(ValueError):
+        SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8", opt_type="gptq-search", device="cpu")
+    assert type(SegmentLinear(8, 8, input_quant_type="int8", weight_quant_type="int8", opt_type="smooth",
+                              device="cpu").optimizer).__name__ == "SmoothOptimizer"
 
 
 def test_quantize_replaces_linears_and_keeps_outputs_close():
@@ -405,3 +407,52 @@ def test_forward_parts_on_the_fake_path_is_the_concatenated_forward():
     with pytest.raises(Exception):
         SegmentLinear(96, 40, seg_mode="weight", chunks=2, input_quant_type="int8", weight_quant_type="int8",
                       device="cpu").optimizer.forward_parts([a, b])
+
+
+@pytest.mark.parametrize("opt_type", ["smooth", "svd"])
+@pytest.mark.parametrize("seg_mode,chunks", [("weight", 1), ("weight", 3), ("input", 2)])
+def test_smooth_and_svd_layers_on_the_fake_path_equal_the_oracle(opt_type, seg_mode, chunks):
+    """trace -> smooth -> calibrate -> forward of the smoothing optimisers (fake quantisation, CPU)
+    against the closed form the oracle builds chunk by chunk: s from the traced maxima, the weight
+    chunk times s split into L1 L2 and a residual, fake-quantised x / s times the fake-quantised
+    residual plus (x / s) L1 L2 (segquant/optimum/optimizer.py:440-517, :640-731)."""
+    import torch
+    from segquant_amd.layers.SegmentLinear import SegmentLinear
+    K, N, M, r, alpha = 48, 36, 10, 4, 0.5
+    g = torch.Generator().manual_seed(11)
+    lin = torch.nn.Linear(K, N)
+    x = torch.randn(M, K, generator=g) * (torch.rand(K, generator=g) * 4 + 0.2)
+    layer = SegmentLinear(K, N, bias=True, seg_mode=seg_mode, chunks=chunks, custom_weight_tensor=lin.weight.data,
+                          custom_bias_tensor=lin.bias.data, input_quant_type="int8", weight_quant_type="int8",
+                          input_quant_args={}, weight_quant_args={}, opt_type=opt_type,
+                          opt_kwargs={"alpha": alpha, **({"low_rank": r} if opt_type == "svd" else {})}, device="cpu")
+    layer.trace(x)
+    layer.smooth()
+    layer.calibrate(x)
+    layer.finish_calibrate()
+    got = layer(x).double().numpy()
+    xn, wn = x.numpy(), lin.weight.data.numpy()
+    want = np.zeros((M, N))
+    ksz, nsz = K // chunks, N // chunks
+    for i in range(chunks):
+        ks = slice(i * ksz, (i + 1) * ksz) if seg_mode == "input" else slice(0, K)
+        ns = slice(0, N) if seg_mode == "input" else slice(i * nsz, (i + 1) * nsz)
+        xc, wc = xn[:, ks], wn[ns, ks]
+        s = O.smooth_factors(np.abs(xc).max(axis=0), np.abs(wc).max(axis=0), alpha)
+        ws = (wc * s).astype(np.float32)
+        xs = (xc / s).astype(np.float32)
+        low = 0.0
+        if opt_type == "svd":
+            l1, l2, res = O.svd_split(ws, r)
+            ws = res.astype(np.float32)
+            low = (xs.astype(np.float64) @ l1.astype(np.float32)) @ l2.astype(np.float32)
+        sx, sw = O.int_scale(float(np.abs(xs).max())), O.int_scale(float(np.abs(ws).max()))
+        want[:, ns] += O.fake_quant_int(xs, sx).astype(np.float64) @ O.fake_quant_int(ws, sw).astype(np.float64).T + low
+    want += lin.bias.data.double().numpy()
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+    ref = lin(x).double().detach().numpy()
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 0.05
+    assert layer.optimizer.fused_available() is False  # no kernels on the CPU
+    with pytest.raises(NotImplementedError):
+        SegmentLinear(K, N, input_quant_type="int8", weight_quant_type="int8", opt_type=opt_type,
+                      opt_kwargs={"search_alpha_config": {"enable": True, "min": 0.1, "max": 0.9, "step": 0.1}}, device="cpu")

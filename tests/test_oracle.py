@@ -444,3 +444,38 @@ def test_int4_column_to_row_repack_against_its_elementwise_definition():
         assert np.array_equal(np.stack([O.unpack_int4(row) for row in got.reshape(out, cols // 2)]), signed)
     with pytest.raises(AssertionError):
         O.repack_int4_cols_to_rows(np.zeros(3, dtype=np.uint8), 3, 2)
+
+
+def test_smooth_factors_and_svd_split_against_what_the_mathematics_fixes():
+    """smooth_factors (optimizer.py:440-457): alpha = 1 gives max_x, alpha = 0 gives 1 / max_w, dead
+    channels give 1, the clamp holds.  svd_split (:640-684): L1 L2 plus the residual reassemble
+    the weight, the residual's Frobenius norm is the energy of the discarded singular values
+    (Eckart-Young), L2 has orthonormal rows, and a weight of rank r leaves no residual.  Smoothing
+    does not change the product: (x / s)(W s)^T == x W^T."""
+    g = np.random.default_rng(21)
+    mx = np.abs(g.standard_normal(40)).astype(np.float32) * 10 + 0.1
+    mw = np.abs(g.standard_normal(40)).astype(np.float32) + 0.05
+    assert np.allclose(O.smooth_factors(mx, mw, 1.0), np.clip(mx, 1e-4, 1e4), rtol=1e-6)
+    assert np.allclose(O.smooth_factors(mx, mw, 0.0), np.clip(1 / mw, 1e-4, 1e4), rtol=1e-6)
+    assert np.allclose(O.smooth_factors(mx, mw, 0.5), np.sqrt(mx.astype(np.float64) / mw), rtol=1e-5)
+    dead = O.smooth_factors(np.float32([0.0, 1e-30, 5.0]), np.float32([1.0, 1.0, 1e-12]), 0.5)
+    assert dead[0] == 1.0 and dead[1] == 1.0 and dead[2] == np.float32(1e4)
+    assert O.smooth_factors(np.float32([1e-9]), np.float32([1e3]), 0.5)[0] == np.float32(1e-4)
+    w = g.standard_normal((24, 40))
+    l1, l2, res = O.svd_split(w, 5)
+    assert l1.shape == (40, 5) and l2.shape == (5, 24) and res.shape == (24, 40)
+    assert np.allclose(res + (l1 @ l2).T, w, atol=1e-12)
+    sv = np.linalg.svd(w, compute_uv=False)
+    assert np.isclose(np.linalg.norm(res), np.sqrt((sv[5:] ** 2).sum()), rtol=1e-10)
+    assert np.allclose(l2 @ l2.T, np.eye(5), atol=1e-12)
+    low = g.standard_normal((24, 3)) @ g.standard_normal((3, 40))
+    assert np.abs(O.svd_split(low, 3)[2]).max() < 1e-10
+    x = g.standard_normal((7, 40))
+    s = O.smooth_factors(mx, mw, 0.5).astype(np.float64)
+    assert np.allclose((x / s) @ (w * s).T, x @ w.T, rtol=1e-12, atol=1e-12)
+    # smooth_svd_linear with a weight that the codes represent exactly and unit scales is x W^T
+    wi = g.integers(-100, 100, size=(24, 40)).astype(np.int8)
+    xi = g.integers(-100, 100, size=(7, 40)).astype(np.float32)
+    ones = np.ones(40, dtype=np.float32)
+    got = O.smooth_svd_linear(xi, ones, wi, [1.0], [1.0], O.FMT_INT8, O.FMT_INT8, l1=l1, l2=l2, bias=np.arange(24))
+    assert np.allclose(got, xi.astype(np.float64) @ wi.T.astype(np.float64) + (xi.astype(np.float64) @ l1) @ l2 + np.arange(24))
