@@ -329,7 +329,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     // finished ranges in: one fp32 tile per workgroup
     bool park = i8 && plain8 && fold && !groups && wide_ok && d->batch == 1 && d->out_dtype != SEGQ_ACC && ws && al(ws, 16);
     auto park_fits = [&](int c) {
-        if (c < FIRST_WIDE_CFG || c > FIRST_WIDE_CFG + 5) return false;
+        if (c < FIRST_WIDE_CFG || c >= NUM_TILE_CFG) return false;
         const TileCfg& t = TILE_CFGS[c];
         const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
         return ws_bytes >= tiles * t.bm * t.bn * 4;
@@ -348,10 +348,25 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
+    // the 8-wave tiles that exist with the finish in output units (low-rank branch, two-way K split)
+    auto tail_tile = [](int c) {
+        const int w = c - FIRST_WIDE_CFG;
+        return w == 0 || w == 1 || w == 3 || w == 6 || w == 7;
+    };
+    if (lowrank && d->tile == 0 && cfg >= FIRST_WIDE_CFG && !tail_tile(cfg)) {
+        cfg = cfg == FIRST_WIDE_CFG + 2 ? FIRST_WIDE_CFG + 1 : FIRST_WIDE_CFG;
+        park = park && park_fits(cfg);
+    }
     // Split K: few tiles and a long contraction.  The K steps of every tile are shared by
-    // `splits` workgroups (grid.y), each writing an fp32 partial result into the workspace;
-    // a second kernel sums them, adds the bias and rounds.  Workspace: the partial results,
-    // then (int8 with several ranges) the parking slots of all those workgroups.
+    // `splits` workgroups (grid.y).
+    //  * Two shares are finished inside the launch: each workgroup leaves its fp32 share in the
+    //    workspace, and the second to arrive adds the two, adds the bias and rounds.  Workspace:
+    //    two tile-sized shares per tile, one word per tile in which the first to arrive leaves the
+    //    launch's stamp (a per-process counter: no clearing between launches, and a fresh workspace
+    //    may hold anything).
+    //  * More shares: each workgroup writes an fp32 partial result, a second kernel sums them in the
+    //    order of the shares.  Workspace: the partial results.
+    // Either way the parking slots of all those workgroups follow (int8 with several ranges).
     int splits = 1;
     int64_t part_bytes = 0;
     {
@@ -363,39 +378,55 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
                                               "a float output, an 8-wave tile and a workspace");
         if (can) {
             int want = 1, scfg = cfg;
-            const bool big_ok0 = !fold2 || park || f8;
+            const bool big_ok = !fold2 || park || f8;  // the 256 x 256 tile, or 256 x 128 with a second register set
+            const int64_t cus = device_cus();
+            auto tiles_of = [&](int c) { return ((d->m + TILE_CFGS[c].bm - 1) / TILE_CFGS[c].bm) * ((d->n + TILE_CFGS[c].bn - 1) / TILE_CFGS[c].bn); };
             if (d->split_k > 1) {
                 want = (int)(d->split_k < total_steps ? d->split_k : total_steps);
-                if (d->tile == 0) scfg = big_ok0 ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
-            } else if (d->tile == 0) {
-                const bool big_ok = !fold2 || park || f8;  // the 256 x 256 tile, or 256 x 128 with a second register set
-                scfg = big_ok ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
-                const TileCfg& t = TILE_CFGS[scfg];
-                const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
-                // measured: 48 tiles x 5 shares beat 192 tiles of 128 x 128 by 19 % (1024 x 15360 x 3072, e4m3),
-                // 96 tiles x 2 shares lose to 192 tiles of 256 x 128 (4096 x 6144 x 1536): the fp32 partial
-                // results and their sum cost what two shares gain
-                // (int8 with several ranges gains nothing: 139 -> 145 us on the same shape)
-                const int64_t cus = device_cus();
-                if (tiles * 4 <= cus && total_steps >= 32 && !(i8 && fold)) {
-                    const int64_t by_cus = cus / tiles, by_steps = total_steps / 8;
-                    want = (int)(by_cus < by_steps ? by_cus : by_steps);
-                    if (want > 16) want = 16;
+                if (d->tile == 0) scfg = big_ok ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
+            } else if (d->tile == 0 && total_steps >= 32 && tiles_of(cfg) * 10 < cus * 9) {
+                // Whole tiles would leave more than a tenth of the CUs idle: look for a big tile and a
+                // number of shares that fill them.  Measured (us, random codes, 256 CUs):
+                //   1024 x 3072, K 13824 twice (DualScale):  e4m3  256x192 x4 99 | 256x256 x5 130 | 128x128 176
+                //                                            int8  256x192 x4 108 | 256x256 x4 125 | 128x128 184
+                //   4096 x 1536, K 6144 twice:               e4m3  256x192 x2 85 | 256x256 x2 94 | 256x128 123
+                // The choice minimises rounds x (K steps per share + fixed cost) x tile area / efficiency:
+                // about 6 steps' worth of prologue and epilogue per workgroup, 8 more for the shares' trip
+                // through memory; big tiles get more out of every byte they stream.
+                auto eff = [](int c) {
+                    const int area = TILE_CFGS[c].bm * TILE_CFGS[c].bn;
+                    return c < FIRST_WIDE_CFG ? 0.5 : area >= 256 * 256 ? 1.0 : area >= 256 * 192 ? 0.95 : area >= 256 * 128 ? 0.85 : 0.7;
+                };
+                auto cost = [&](int c, int64_t s_) {
+                    const int64_t wgs = tiles_of(c) * s_;
+                    return (double)((wgs + cus - 1) / cus) * ((double)total_steps / s_ + 6.0 + (s_ > 1 ? 8.0 : 0.0)) *
+                           TILE_CFGS[c].bm * TILE_CFGS[c].bn / eff(c);
+                };
+                const int cands[3] = {FIRST_WIDE_CFG + 6, FIRST_WIDE_CFG, FIRST_WIDE_CFG + 7};
+                double best = cost(cfg, 1);
+                for (int i = 0; i < (big_ok ? 3 : 1); ++i) {
+                    const int c = big_ok ? cands[i] : FIRST_WIDE_CFG + 1;
+                    int64_t s_ = cus / tiles_of(c);
+                    if (s_ > total_steps / 8) s_ = total_steps / 8;
+                    if (s_ > 16) s_ = 16;
+                    if (s_ < 2) continue;
+                    if (cost(c, s_) < best) { best = cost(c, s_); scfg = c; want = (int)s_; }
                 }
             }
             const TileCfg& t = TILE_CFGS[scfg];
-            const int64_t tiles = ((d->m + t.bm - 1) / t.bm) * ((d->n + t.bn - 1) / t.bn);
+            const int64_t tiles = tiles_of(scfg);
             const bool need_park = i8 && fold && scfg != FIRST_WIDE_CFG + 1 && scfg != FIRST_WIDE_CFG + 2 && scfg != FIRST_WIDE_CFG + 3;
-            auto bytes_for = [&](int s_) {
-                const int64_t pb = (((int64_t)s_ * d->m * d->n * 4) + 255) & ~(int64_t)255;
-                return pb + (need_park || park ? (int64_t)s_ * tiles * t.bm * t.bn * 4 : 0);
+            auto shares_for = [&](int s_) {
+                if (s_ == 2 && tail_tile(scfg)) return tiles * 2 * t.bm * t.bn * 4 + ((tiles * 4 + 255) & ~(int64_t)255);
+                return (((int64_t)s_ * d->m * d->n * 4) + 255) & ~(int64_t)255;
             };
+            auto bytes_for = [&](int s_) { return shares_for(s_) + (need_park || park ? (int64_t)s_ * tiles * t.bm * t.bn * 4 : 0); };
             while (want > 1 && bytes_for(want) > ws_bytes) --want;
             if (d->split_k > 1 && want < 2) return fail(SEGQ_ERR_ARG, "segq_gemm: workspace too small for split_k");
             if (want > 1) {
                 splits = want;
                 cfg = scfg;
-                part_bytes = (((int64_t)splits * d->m * d->n * 4) + 255) & ~(int64_t)255;
+                part_bytes = shares_for(splits);
                 park = (need_park || park) && i8 && fold;
             }
         }
@@ -443,6 +474,16 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
     p.vec_store = ((d->ldo * osz) % (4 * osz) == 0) && ((d->batch_stride_out * osz) % (4 * osz) == 0) && al(d->out, 4 * osz);
     p.vec_store16 = osz == 2 && d->ldo % 8 == 0 && d->batch_stride_out % 8 == 0 && al(d->out, 16);
+    if (splits == 2 && tail_tile(cfg)) {
+        p.splits = 2;
+        p.part = static_cast<float*>(d->workspace);
+        const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+        p.arrived = reinterpret_cast<unsigned int*>(static_cast<uint8_t*>(d->workspace) + tiles * 2 * c.bm * c.bn * 4);
+        p.bsA = p.bsB = p.bsC = p.bsSx = p.bsSw = 0;  // blockIdx.y counts shares here, not problems
+        static unsigned int g_stamp = 0x5e690000u;
+        p.stamp = __atomic_add_fetch(&g_stamp, 1u, __ATOMIC_RELAXED);
+        return i8 ? launch_gemm_i8(p, cfg, fold, 2, st) : launch_gemm_f8(p, cfg, fold, 2, st);
+    }
     if (splits > 1) {
         p.splits = splits;
         p.C = d->workspace;

@@ -53,6 +53,10 @@ struct GemmParams {
     int32_t splits;       // > 1: grid.y workgroups share the K steps of a tile (gemm_pipe_kernel only)
     int32_t pad_;
     float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
+    float* part;          // splits == 2 finished in the launch: two tile-sized fp32 shares per tile (or null)
+    unsigned int* arrived;  // ... and one word per tile: the first of the two workgroups leaves `stamp` there
+    unsigned int stamp;     // differs from launch to launch
+    unsigned int pad4_;
     const float* grw;     // group-wise de-quantisation factors [K / 128][grw_gs], or null
     int64_t grw_gs;
     const uint16_t* lr_t;   // low-rank branch: T (M x lr_rank) and L2^T (N x lr_rank) in the output's 16-bit dtype, or null
@@ -439,13 +443,14 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
 
 // ---- host-side launch of one (format, tile, fold) instance -------------------
 struct TileCfg { int bm, bn, wgm, wgn; };
-constexpr int NUM_TILE_CFG = 16;
+constexpr int NUM_TILE_CFG = 18;
 constexpr int FIRST_BIG_CFG = 8;    // two retired ids (a 4-wave 256 x 256 kernel that no shape profited from)
-constexpr int FIRST_WIDE_CFG = 10;  // six ids: the 8-wave kernels (segq_gemm_wide.h); the last two plain int8 only
+constexpr int FIRST_WIDE_CFG = 10;  // eight ids: the 8-wave kernels (segq_gemm_wide.h)
 constexpr TileCfg TILE_CFGS[NUM_TILE_CFG] = {
     {256, 256, 2, 2}, {256, 128, 2, 2}, {128, 128, 2, 2}, {64, 128, 2, 2}, {128, 256, 2, 2},
     {256, 256, 2, 4}, {256, 256, 4, 2}, {256, 128, 4, 2}, {256, 256, 2, 2}, {256, 256, 2, 2},
     {256, 256, 4, 2}, {256, 128, 4, 2}, {128, 256, 2, 4}, {128, 128, 2, 4}, {192, 288, 4, 2}, {288, 192, 2, 4},
+    {256, 192, 4, 2}, {192, 256, 2, 4},
 };
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>

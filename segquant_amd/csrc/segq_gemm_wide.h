@@ -513,7 +513,7 @@ __device__ __forceinline__ void lowrank_accumulate(const GemmParams& p, v4f (&of
 // s_waitcnt immediate for "vmcnt(n) lgkmcnt(0)" on gfx9-family encodings
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }
 
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmParams p) {
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -573,11 +573,22 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     const int wm = wave % WGM, wn = wave / WGM;
     const int lrow = lane & 15, lgrp = lane >> 4;
 
-    int bid = blockIdx.x;
+    // Workgroups are dealt to the eight XCDs in turn, each with an L2 of its own.  Every XCD gets a
+    // run of consecutive tiles (with a K split: of consecutive (share, tile) pairs), so that its
+    // workgroups stream few distinct operand panels and its L2 serves most of their requests.
+    int bid = blockIdx.x, zy = blockIdx.y;
     {
         const int nb = p.tiles_m * p.tiles_n;
-        if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+        if (p.splits > 1) {
+            const int total = nb * p.splits, lin = zy * nb + bid, q = total >> 3, r = total & 7, x = lin & 7;
+            const int v = x * q + min(x, r) + (lin >> 3);
+            zy = v / nb;
+            bid = v - zy * nb;
+        } else if ((nb & 7) == 0) {
+            bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+        }
     }
+    const int tile_id = bid;  // names this tile's room in the workspaces
     int tile_m, tile_n;
     {
         const int gsz = p.group_m * p.tiles_n;
@@ -589,7 +600,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         tile_n = in_g / rows_in_group;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int64_t z = blockIdx.y;
+    const int64_t z = zy;
     const uint8_t* const Ab = p.A + z * p.bsA;
     const uint8_t* const A2b = p.A2 ? p.A2 + z * p.bsA : nullptr;
     const uint8_t* const Bb = p.B + z * p.bsB;
@@ -683,7 +694,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     };
     const int m_base = m0 + wm * WM + lrow;
     const int n_base = n0 + wn * WN + 4 * lgrp;
-    v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (BM * BN / 4) + tid : nullptr;
+    v4f* const slot = PARK ? reinterpret_cast<v4f*>(p.park) + ((int64_t)zy * gridDim.x + tile_id) * (BM * BN / 4) + tid : nullptr;
     auto park = [&](int r) __attribute__((always_inline)) {
         if constexpr (PARK) {
             if (r < r_last) {
@@ -781,8 +792,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     for (int i = 0; i < p.nr; ++i) steps += (p.r[i].k1 - p.r[i].k0) / BK;
     int lr = 0, skip = 0;  // this workgroup's first step: `skip` steps into range lr
     if (p.splits > 1) {
-        skip = (int)((int64_t)steps * (int)blockIdx.y / p.splits);
-        steps = (int)((int64_t)steps * ((int)blockIdx.y + 1) / p.splits) - skip;
+        skip = (int)((int64_t)steps * zy / p.splits);
+        steps = (int)((int64_t)steps * (zy + 1) / p.splits) - skip;
         while (lr + 1 < p.nr && skip >= (p.r[lr].k1 - p.r[lr].k0) / BK) {
             skip -= (p.r[lr].k1 - p.r[lr].k0) / BK;
             ++lr;
@@ -1062,28 +1073,79 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     if constexpr (ACCF) {
         if (dirty) fold(cr);
     }
-    if (p.lr_rank > 0) {
-        // Low-rank branch (out += T L2): the sums go to output units first (1 / (sx sw) of the range
-        // they are in units of, from the vectors parked in LDS), the low-rank product joins them in
-        // fp32 on the matrix cores, and the epilogue then only adds the bias and rounds once.
+    if constexpr (FINISH) {
+        // FINISH instances serve the launches that finish in output units (the others do not pay for
+        // the registers of it): the low-rank branch and a tile split in two along K.  The sums are
+        // scaled first (1 / (sx sw) of the range they are in units of, from the vectors parked in LDS); then
+        //  * a tile split in two along K: the two workgroups meet in the workspace (below);
+        //  * low-rank branch (out += T L2): the product joins in fp32 on the matrix cores;
+        // and the epilogue only adds the bias and the addend and rounds once.
         v4f of[TN][TM];
         [[maybe_unused]] const bool parked = r_begin < r_last;
+        constexpr int CH = 8;  // blocks whose loads are in flight at once (registers: the sums are still live)
 #pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const float rx = ACCF ? 1.0f : epi[wm * WM + b * 16 + lrow];
+        for (int c0 = 0; c0 < TN * TM; c0 += CH) {
+            [[maybe_unused]] v4f old[CH];
+            if constexpr (PARK) {
 #pragma unroll
-            for (int a = 0; a < TN; ++a) {
-                v4f t;
-                if constexpr (HASF) t = accf[a][b];
-                else t = __builtin_convertvector(acc[a][b], v4f);
-                if constexpr (PARK) {
-                    if (parked) t += slot[(a * TM + b) * NT];
+                for (int i = 0; i < CH; ++i)
+                    if (c0 + i < TN * TM) old[i] = parked ? slot[(c0 + i) * NT] : v4f{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                if (c0 + i < TN * TM) {
+                    const int a = (c0 + i) / TM, b = (c0 + i) % TM;
+                    v4f t;
+                    if constexpr (HASF) t = accf[a][b];
+                    else t = __builtin_convertvector(acc[a][b], v4f);
+                    if constexpr (PARK) t += old[i];
+                    if constexpr (!ACCF)
+                        t = t * (*reinterpret_cast<const v4f*>(epi + BM + wn * WN + a * 16 + 4 * lgrp) * epi[wm * WM + b * 16 + lrow]);
+                    of[a][b] = t;
                 }
-                if constexpr (!ACCF) t = t * (*reinterpret_cast<const v4f*>(epi + BM + wn * WN + a * 16 + 4 * lgrp) * rx);
-                of[a][b] = t;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (p.part) {
+            // Two workgroups share a tile.  Each leaves its share in the workspace and counts itself in;
+            // the one that finds the other counted adds that share to its own (a + b = b + a: the result
+            // does not depend on who came last) and finishes the tile.  The two can sit on different
+            // XCDs, whose L2 caches do not see each other's lines, so the shares are written through
+            // and read past the caches (agent scope: what the compiler emits for a relaxed agent-scope
+            // atomic, but 16 bytes per lane: 1 KB contiguous per wave and instruction).
+            using v4u = __attribute__((ext_vector_type(4))) unsigned int;
+            constexpr int AGENT = 16;  // the cache-policy bit for agent scope
+            constexpr int SHARE = BM * BN * 4;
+            const int my = zy;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                reinterpret_cast<uint8_t*>(p.part) + (int64_t)tile_id * 2 * SHARE, 0, 2 * SHARE, 0x00020000);
+#pragma unroll
+            for (int i = 0; i < TN * TM; ++i)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, of[i / TM][i % TM]), rs, tid * 16, my * SHARE + i * NT * 16, AGENT);
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));  // this wave's stores have reached memory
+            __syncthreads();                                  // ... and so have the other waves'
+            int* const flag = reinterpret_cast<int*>(epi);    // (1 / sx of row 0: no longer needed)
+            if (tid == 0) {
+                // the launch's own stamp instead of a count: whatever the word held before (an earlier
+                // launch's stamp, or anything at all in a fresh workspace) reads as "nobody yet"
+                const unsigned before = __hip_atomic_exchange(p.arrived + tile_id, p.stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = before == p.stamp;
+            }
+            __syncthreads();
+            if (!*flag) return;
+#pragma unroll
+            for (int c0 = 0; c0 < TN * TM; c0 += CH) {
+                v4u other[CH];
+#pragma unroll
+                for (int i = 0; i < CH; ++i)
+                    if (c0 + i < TN * TM)
+                        other[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, tid * 16, (1 - my) * SHARE + (c0 + i) * NT * 16, AGENT);
+#pragma unroll
+                for (int i = 0; i < CH; ++i)
+                    if (c0 + i < TN * TM) of[(c0 + i) / TM][(c0 + i) % TM] += __builtin_bit_cast(v4f, other[i]);
             }
         }
-        lowrank_accumulate<TM, TN>(p, of, m0 + wm * WM, n0 + wn * WN, lane);
+        if (p.lr_rank > 0) lowrank_accumulate<TM, TN>(p, of, m0 + wm * WM, n0 + wn * WN, lane);
         wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, true>(p, of, of, smem, z, m0, n0, wave, lane, r_epi, epi);
         return;
     }
@@ -1126,9 +1188,9 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 }
 
 // wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false>
 int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
-    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK>;
+    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK, FINISH>;
     // the stages, the epilogue's vectors, and the ring of group factors
     constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4 + (GRP ? 4 * BN * 4 : 0);
     static unsigned long long attr_done = 0;
@@ -1140,9 +1202,10 @@ int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 
 template <int FMT, bool B4>
 int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t batch, hipStream_t st) {
+    const bool tail = p.lr_rank > 0 || p.part;  // finishes in output units: the FINISH instances (tail_tile() says which exist)
     if constexpr (!B4 && FMT == GEMM_I8) {
         if (p.grw) {  // group-wise factors (the host has checked: plain codes, K ranges in whole steps)
-            if (asel) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need plain codes");
+            if (asel || tail) return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors need plain codes, and serve no low-rank branch");
             switch (wcfg) {
                 case 0: case 1:
                     return fold ? launch_pipe_instance<256, 128, 4, 2, FMT, true, 2, true>(p, batch, st)
@@ -1157,47 +1220,64 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: group factors run on the 256x128, 128x256 and 128x128 tiles of eight waves");
         }
     }
+// a tile that exists with and without the tail / without only
+#define SEGQ_PIPE2(BM_, BN_, WGM_, WGN_, FOLD_, PARK_)                                                               \
+    return tail ? launch_pipe_instance<BM_, BN_, WGM_, WGN_, FMT, FOLD_, 2, false, PARK_, true>(p, batch, st)        \
+                : launch_pipe_instance<BM_, BN_, WGM_, WGN_, FMT, FOLD_, 2, false, PARK_, false>(p, batch, st)
+#define SEGQ_PIPE1(BM_, BN_, WGM_, WGN_, FOLD_, PARK_)                                                               \
+    if (tail) break;                                                                                                 \
+    return launch_pipe_instance<BM_, BN_, WGM_, WGN_, FMT, FOLD_, 2, false, PARK_, false>(p, batch, st)
     if constexpr (!B4) {
         constexpr bool F8W = FMT == GEMM_F8;  // the e4m3 schedule wants three or more column blocks per wave
         if (!asel) {  // plain 8-bit operands, both straight to LDS: the software-pipelined kernel
             if (!fold) {
                 switch (wcfg) {
-                    case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2>(p, batch, st);
-                    case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, false, 2>(p, batch, st);
-                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, false, 2>(p, batch, st);
-                    case 3: return launch_pipe_instance<128, 128, F8W ? 4 : 2, F8W ? 2 : 4, FMT, false, 2>(p, batch, st);
-                    case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, false, 2>(p, batch, st);
-                    case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, false, 2>(p, batch, st);
+                    case 0: SEGQ_PIPE2(256, 256, 4, 2, false, false);
+                    case 1: SEGQ_PIPE2(256, 128, 4, 2, false, false);
+                    case 2: SEGQ_PIPE1(128, 256, 2, 4, false, false);
+                    case 3: SEGQ_PIPE2(128, 128, (F8W ? 4 : 2), (F8W ? 2 : 4), false, false);
+                    case 4: SEGQ_PIPE1(192, 288, 4, 2, false, false);
+                    case 5: SEGQ_PIPE1(288, 192, 2, 4, false, false);
+                    case 6: SEGQ_PIPE2(256, 192, 4, 2, false, false);
+                    case 7: SEGQ_PIPE2(192, 256, 2, 4, false, false);
                 }
             } else if constexpr (F8W) {  // fp32 accumulators are rescaled in place: every tile serves several ranges
                 switch (wcfg) {
-                    case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, true, 2>(p, batch, st);
-                    case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2>(p, batch, st);
-                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2>(p, batch, st);
-                    case 3: return launch_pipe_instance<128, 128, 4, 2, FMT, true, 2>(p, batch, st);
-                    case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, true, 2>(p, batch, st);
-                    case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, true, 2>(p, batch, st);
+                    case 0: SEGQ_PIPE2(256, 256, 4, 2, true, false);
+                    case 1: SEGQ_PIPE2(256, 128, 4, 2, true, false);
+                    case 2: SEGQ_PIPE1(128, 256, 2, 4, true, false);
+                    case 3: SEGQ_PIPE2(128, 128, 4, 2, true, false);
+                    case 4: SEGQ_PIPE1(192, 288, 4, 2, true, false);
+                    case 5: SEGQ_PIPE1(288, 192, 2, 4, true, false);
+                    case 6: SEGQ_PIPE2(256, 192, 4, 2, true, false);
+                    case 7: SEGQ_PIPE2(192, 256, 2, 4, true, false);
                 }
             } else if (p.park) {  // int8, several ranges, a workspace to park finished ranges in: every tile
                 if constexpr (!F8W) {
                     switch (wcfg) {
-                        case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, true, 2, false, true>(p, batch, st);
-                        case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2, false, true>(p, batch, st);
-                        case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2, false, true>(p, batch, st);
-                        case 3: return launch_pipe_instance<128, 128, 2, 4, FMT, true, 2, false, true>(p, batch, st);
-                        case 4: return launch_pipe_instance<192, 288, 4, 2, FMT, true, 2, false, true>(p, batch, st);
-                        case 5: return launch_pipe_instance<288, 192, 2, 4, FMT, true, 2, false, true>(p, batch, st);
+                        case 0: SEGQ_PIPE2(256, 256, 4, 2, true, true);
+                        case 1: SEGQ_PIPE2(256, 128, 4, 2, true, true);
+                        case 2: SEGQ_PIPE1(128, 256, 2, 4, true, true);
+                        case 3: SEGQ_PIPE2(128, 128, 2, 4, true, true);
+                        case 4: SEGQ_PIPE1(192, 288, 4, 2, true, true);
+                        case 5: SEGQ_PIPE1(288, 192, 2, 4, true, true);
+                        case 6: SEGQ_PIPE2(256, 192, 4, 2, true, true);
+                        case 7: SEGQ_PIPE2(192, 256, 2, 4, true, true);
                     }
                 }
             } else {
                 switch (wcfg) {
-                    case 0: case 1: return launch_pipe_instance<256, 128, 4, 2, FMT, true, 2>(p, batch, st);
-                    case 2: return launch_pipe_instance<128, 256, 2, 4, FMT, true, 2>(p, batch, st);
-                    case 3: return launch_pipe_instance<128, 128, F8W ? 4 : 2, F8W ? 2 : 4, FMT, true, 2>(p, batch, st);
+                    case 0: case 1: SEGQ_PIPE2(256, 128, 4, 2, true, false);
+                    case 2: SEGQ_PIPE1(128, 256, 2, 4, true, false);
+                    case 3: SEGQ_PIPE2(128, 128, (F8W ? 4 : 2), (F8W ? 2 : 4), true, false);
                 }
             }
         }
     }
+#undef SEGQ_PIPE1
+#undef SEGQ_PIPE2
+    if (tail)
+        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: tile %d finishes neither a low-rank branch nor a two-way K split", wcfg + FIRST_WIDE_CFG + 1);
 #define SEGQ_WIDE(BM_, BN_, WGM_, WGN_, FOLD_)                                                          \
     return asel ? launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, true>(p, batch, st)       \
                 : launch_wide_instance<BM_, BN_, WGM_, WGN_, FMT, B4, FOLD_, false>(p, batch, st)

@@ -247,7 +247,7 @@ def gemm_workspace_bytes(g) -> int:
 
 # tile ids of the 8-wave kernels (segq_gemm_desc.tile) -> rows x columns of the output tile
 TILE_SHAPES = {1: "256x256", 2: "256x128", 3: "128x128", 4: "64x128", 5: "128x256", 6: "256x256", 7: "256x256", 8: "256x128",
-               11: "256x256", 12: "256x128", 13: "128x256", 14: "128x128", 15: "192x288", 16: "288x192"}
+               11: "256x256", 12: "256x128", 13: "128x256", 14: "128x128", 15: "192x288", 16: "288x192", 17: "256x192", 18: "192x256"}
 
 
 def gemm_plan(g, workspace: Optional[torch.Tensor] = None) -> dict:
@@ -283,17 +283,11 @@ def park_bytes(m: int, n: int) -> int:
 def split_bytes(m: int, n: int, splits: int = 16, park: bool = False) -> int:
     """Workspace for a GEMM whose K steps are shared by up to ``splits`` workgroups per
     tile: the fp32 partial results and, for int8 with several ranges (``park``), the
-    parking room of all those workgroups."""
-    return splits * (4 * m * n + (park_bytes(m, n) if park else 0)) + 256
+    parking room of all those workgroups.  (Two shares are kept as whole tiles, with one
+    arrival counter per tile behind them; ``gemm_workspace_bytes`` gives the exact figure.)"""
+    counters = 4 * -(-m // 128) * -(-n // 128) + 512
+    return splits * park_bytes(m, n) * (2 if park else 1) + counters
 
-
-def auto_splits(m: int, n: int, k_steps: int) -> int:
-    """How many shares the library's own rule would take for an (m, n) problem of
-    ``k_steps`` 128-byte K steps (0: it would not split), to size the workspace with."""
-    tiles = -(-m // 256) * -(-n // 256)
-    if tiles * 4 > 256 or k_steps < 32:
-        return 0
-    return max(0, min(256 // tiles, k_steps // 8, 16))
 
 
 def gemm(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], **kw) -> torch.Tensor:

@@ -374,14 +374,12 @@ class DefaultOptimizer(BaseOptimizer):
         #    expanded to int8 once per launch and the int8 kernels run; with few tokens reading half
         #    the weight bytes matters more (measured, K 1280, N 10240: 161 -> 119 us at 8192 tokens,
         #    no gain at 2048).  Group-wise scales run on the int8 kernels only: always lend.
-        #  * int8 with several ranges (K segments, DualScale) and many tokens: room to park the
-        #    finished ranges' sums keeps the big tiles (4608 x 15360 x 3072, three ranges:
-        #    441 -> 383 us; 9216 tokens: 1044 -> 756 us; no gain at 1024 tokens).
-        #  * few tiles and a long K (config 5 at 1024 tokens): room to share the K steps of a tile
-        #    between workgroups.
+        #  * 8-bit weights: always.  int8 with several ranges (K segments, DualScale) parks the
+        #    finished ranges' sums there and keeps the big tiles (4608 x 15360 x 3072, three ranges:
+        #    441 -> 383 us; 9216 tokens: 1044 -> 756 us); few tiles and a long K share the K steps of
+        #    a tile between workgroups (1024 x 15360 x 3072: 162 -> 108 us int8, 135 -> 98 us e4m3).
         int4 = plan["fw"] == ops.FMT_INT4
-        int8_ranges = plan["fa"] == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1
-        lend = (M >= 3072 or gdq is not None) if int4 else (M >= 2048 or not int8_ranges)
+        lend = (M >= 3072 or gdq is not None) if int4 else True
         ws = None
         if lend:
             need = plan.setdefault("ws_need", {}).get(M)
@@ -467,9 +465,8 @@ class DefaultOptimizer(BaseOptimizer):
         g = ops.gemm_desc(codes, plan["w"], ranges, m=M, n=N, a_fmt=fa, b_fmt=plan["fw"], out_dtype=dt, lda=K,
                           ldb=K // 2 if plan["fw"] == ops.FMT_INT4 else K, bias=bias, a_neg=codes_neg)
         int4 = plan["fw"] == ops.FMT_INT4
-        int8_ranges = fa == plan["fw"] == ops.FMT_INT8 and len(ranges) > 1
         ws = None
-        if (M >= 3072) if int4 else (M >= 2048 or not int8_ranges):
+        if M >= 3072 or not int4:
             need = plan.setdefault("ws_need", {}).get(M)
             if need is None:
                 need = plan["ws_need"][M] = ops.gemm_workspace_bytes(g)

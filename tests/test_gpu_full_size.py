@@ -200,12 +200,11 @@ def test_full_size_config5_three_ranges_against_closed_form(ops, M, fmt, lend):
     sw, bias = torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
     s0d, sxd, sx2d, swd = (t.to(DEV) for t in (s0, sx, sx2, sw))
     rg = [ops.Range(0, K0, s0d, swd, 0, 0, 1), ops.Range(K0, K1, sxd, swd, 0, 1, 1), ops.Range(K0, K1, sx2d, swd, 1, 1, 1)]
+    gd = ops.gemm_desc(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, bias=bias.to(DEV), a_neg=a2d)
     ws = None
-    if lend:
-        nbytes = max(ops.park_bytes(M, N), ops.split_bytes(M, N, max(ops.auto_splits(M, N, (K0 + 2 * K1) // 128), 1)))
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
-    out = ops.gemm(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.float32, lda=K, ldb=K, bias=bias.to(DEV),
-                   a_neg=a2d, workspace=ws)
+    if lend:  # exactly what the library says it can use (parking room, K shares)
+        ws = torch.empty(max(ops.gemm_workspace_bytes(gd), 16), dtype=torch.uint8, device=DEV)
+    out = ops.gemm_launch(gd, ws)
     got = out.cpu().numpy().astype(np.float64)
     av, a2v, bv = O.code_values(a, fmt), O.code_values(a2, fmt), O.code_values(b, fmt)
     s0n, sxn, sx2n, swn, bn = (t.numpy().astype(np.float64) for t in (s0, sx, sx2, sw, bias))

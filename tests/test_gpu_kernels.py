@@ -221,7 +221,7 @@ def test_gemm_raw_accumulators(ops, tile, fa, fb, M, N, K):
         assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
 
 
-WIDE_TILES = [11, 12, 13, 14, 15, 16]   # the 8-wave kernels; 15 and 16 (192x288, 288x192) serve plain 8-bit codes only
+WIDE_TILES = [11, 12, 13, 14, 15, 16, 17, 18]   # the 8-wave kernels; 15 to 18 (192x288, 288x192, 256x192, 192x256) serve plain 8-bit codes only
 
 
 def _bf16_ulp(ref):
@@ -353,7 +353,7 @@ def test_gemm_int4_weights_expanded_into_a_lent_workspace(ops):
 
 
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
-@pytest.mark.parametrize("tile", [0, 11, 12, 14, 16])
+@pytest.mark.parametrize("tile", [0, 11, 12, 14, 16, 17, 18])
 def test_gemm_split_k(ops, fmt, tile):
     """The K steps of every tile shared by 2..7 workgroups, shares that begin and end inside
     ranges, one range and three (K segments + a two-tensor DualScale segment), ragged M and N,
@@ -396,7 +396,41 @@ def test_gemm_split_k(ops, fmt, tile):
         ops.gemm(ad, bd, one, out_dtype=torch.float32, split_k=2, workspace=ws, tile=3, m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K)
 
 
-@pytest.mark.parametrize("tile", [0, 11, 12, 13, 14, 15, 16])
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("tile", [11, 12, 14, 17, 18])
+def test_gemm_two_shares_finished_in_the_launch(ops, fmt, tile):
+    """A tile split in two along K is finished by whichever of its two workgroups arrives second
+    (no second kernel): equal to the unsplit launch up to fp32 summation order, the same bits on
+    every run (a + b = b + a), with bias, addend and a bf16 output, over many tiles, a workspace
+    that is reused dirty, and a workspace of exactly the size the library asks for."""
+    M, N, K = 1024, 1152, 2048
+    a, b = _rand_codes((M, K), fmt, 71), _rand_codes((N, K), fmt, 72)
+    ad, bd = _to_dev_codes(a, fmt), _to_dev_codes(b, fmt)
+    g = torch.Generator().manual_seed(73)
+    sx, sw, bias = torch.rand(M, generator=g) + 0.5, torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    add = torch.randn(M, N, generator=g).to(torch.bfloat16).to(DEV)
+    rg = [ops.Range(0, 768, sx.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(768, K - 768, sx.to(DEV) * 1.5, sw.to(DEV), 0, 1, 1)]
+    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, bias=bias.to(DEV), tile=tile, addend=add, out_dtype=torch.bfloat16)
+    gd = ops.gemm_desc(ad, bd, rg, split_k=2, **kw)
+    big = torch.empty(64 << 20, dtype=torch.uint8, device=DEV)
+    plan = ops.gemm_plan(gd, big)
+    assert plan["splits"] == 2 and plan["tile"] == tile
+    need = ops.gemm_workspace_bytes(gd)
+    shape = ops.TILE_SHAPES[tile].split("x")
+    tiles = -(-M // int(shape[0])) * -(-N // int(shape[1]))
+    assert need >= tiles * 2 * int(shape[0]) * int(shape[1]) * 4 + tiles * 4
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)  # dirty: the counters are cleared by the launch
+    ref = ops.gemm(ad, bd, rg, split_k=1, workspace=big, **kw)
+    outs = [ops.gemm(ad, bd, rg, split_k=2, workspace=ws, **kw).clone() for _ in range(4)]
+    for o in outs:
+        assert torch.equal(o, outs[0])
+    assert (outs[0].float() - ref.float()).abs().max().item() <= 2.0 ** -7 * ref.float().abs().max().item()
+    o32 = ops.gemm(ad, bd, rg, split_k=2, workspace=ws, **{**kw, "out_dtype": torch.float32, "addend": None})
+    r32 = ops.gemm(ad, bd, rg, split_k=1, workspace=big, **{**kw, "out_dtype": torch.float32, "addend": None})
+    assert (o32 - r32).abs().max().item() <= (3e-6 if fmt == O.FMT_INT8 else 3e-4) * r32.abs().max().item()
+
+
+@pytest.mark.parametrize("tile", [0, 11, 12, 13, 14, 15, 16, 17, 18])
 def test_gemm_int8_ranges_parked_in_a_lent_workspace(ops, tile):
     """int8 with K segments and a two-tensor DualScale segment on every 8-wave tile: the sums of
     finished ranges wait in the caller's workspace instead of a second register set.  Checked
@@ -974,9 +1008,14 @@ def test_gemm_low_rank_branch_in_the_epilogue(ops, fmt, dt, ranges, lend):
         l2t = (torch.randn(N, rank, generator=tg) * 0.5).to(TDT[dt])
         want = base + bias.numpy().astype(np.float64) + t_lr.double().numpy() @ l2t.double().numpy().T
         ws = torch.empty(ops.park_bytes(M, N), dtype=torch.uint8, device=DEV) if lend else None
-        for tile in (0, 11, 12, 13, 14, 15, 16):
-            if ranges == 3 and fmt == O.FMT_INT8 and not lend and tile in (11, 15, 16):
+        for tile in (0, 11, 12, 13, 14, 15, 16, 17, 18):
+            if ranges == 3 and fmt == O.FMT_INT8 and not lend and tile in (11, 15, 16, 17, 18):
                 continue  # these tiles have no second accumulator set: they need the workspace
+            if tile in (13, 15, 16):  # tiles that are not built with the finish in output units
+                with pytest.raises(RuntimeError):
+                    ops.gemm(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=K, bias=bias.to(DEV),
+                             a_neg=a2d if ranges == 3 else None, tile=tile, workspace=ws, lowrank=(t_lr.to(DEV), l2t.to(DEV)))
+                continue
             out = ops.gemm(ad, bd, rg, m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=K, bias=bias.to(DEV),
                            a_neg=a2d if ranges == 3 else None, tile=tile, workspace=ws, lowrank=(t_lr.to(DEV), l2t.to(DEV)))
             got = out.float().cpu().numpy().astype(np.float64)

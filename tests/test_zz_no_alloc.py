@@ -53,14 +53,14 @@ def _both(ops, make_desc):
     return want, g2[1], need
 
 
-def _split_case(ops, M, N, K, fmt, seed):
+def _split_case(ops, M, N, K, fmt, seed, split_k=0):
     a, b = _codes((M, K), fmt, seed), _codes((N, K), fmt, seed + 1)
     g = torch.Generator().manual_seed(seed)
     sx = (torch.rand(M, generator=g) + 0.5).to(DEV)
     sw = (torch.rand(N, generator=g) + 0.5).to(DEV)
     bias = torch.randn(N, generator=g).to(DEV)
     return lambda: ops.gemm_desc(a, b, [ops.Range(0, K, sx, sw, 0, 1, 1)], m=M, n=N, a_fmt=fmt, b_fmt=fmt,
-                                 out_dtype=torch.bfloat16, lda=K, ldb=K, bias=bias)
+                                 out_dtype=torch.bfloat16, lda=K, ldb=K, bias=bias, split_k=split_k)
 
 
 def _park_case(ops, M, N, K0, K1, seed):
@@ -88,8 +88,9 @@ def test_noalloc_matches_the_lent_workspace_twice_in_a_row(ops):
     assert L.lib().segq_noalloc_scratch_bytes() == 64 << 20
     cases = [
         # few tiles, long K: the K steps of a tile are shared by several workgroups (fp32 partial results)
-        ("split e4m3", _split_case(ops, 512, 1024, 8192, O.FMT_E4M3, 1), _split_case(ops, 384, 512, 4096, O.FMT_E4M3, 5)),
-        ("split int8", _split_case(ops, 512, 768, 8192, O.FMT_INT8, 11), _split_case(ops, 200, 256, 4096, O.FMT_INT8, 15)),
+        # (the library's own choice of shares, then shares asked for: four, and two, which meet inside the launch)
+        ("split e4m3", _split_case(ops, 512, 1024, 8192, O.FMT_E4M3, 1), _split_case(ops, 384, 512, 4096, O.FMT_E4M3, 5, 4)),
+        ("split int8", _split_case(ops, 512, 768, 8192, O.FMT_INT8, 11), _split_case(ops, 200, 256, 4096, O.FMT_INT8, 15, 2)),
         # int8 with three ranges: finished ranges parked as fp32
         ("park", _park_case(ops, 1536, 1408, 256, 512, 21), _park_case(ops, 1300, 1200, 128, 256, 25)),
         # int4 weights expanded to int8
