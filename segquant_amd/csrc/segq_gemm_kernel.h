@@ -282,8 +282,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
                         acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[a], fa[b], acc[a][b], 0, 0, 0);
             }
         } else {
-            const int off0 = ((2 * lgrp) ^ f_sw) << 4;
-            const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
+            // (K slot g of the MFMA gets 16-byte pieces g and 4 + g of the step, for both operands:
+            // the int8 path's conflict-free read pattern)
+            const int off0 = (lgrp ^ f_sw) << 4;
+            const int off1 = ((4 + lgrp) ^ f_sw) << 4;
             v8i fa[TM], fb[TN];
 #pragma unroll
             for (int t = 0; t < TM; ++t) {

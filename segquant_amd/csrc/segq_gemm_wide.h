@@ -363,8 +363,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_wide_kernel(const GemmPara
                         acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[a], fa[b], acc[a][b], 0, 0, 0);
             }
         } else {
-            const int off0 = ((2 * lgrp) ^ f_sw) << 4;
-            const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
+            // (K slot g of the MFMA gets 16-byte pieces g and 4 + g of the step, for both operands:
+            // the int8 path's conflict-free read pattern)
+            const int off0 = (lgrp ^ f_sw) << 4;
+            const int off1 = ((4 + lgrp) ^ f_sw) << 4;
             v8i fa[TM], fb[TN];
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
@@ -668,8 +670,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     v8i fa8[S8 ? TM : 1], fb8[S8 ? TN : 1];
     auto frag8 = [&](int buf, int i) {  // fragment i of the step in buffer buf: 0 .. TM-1 activations, then weights
       if constexpr (S8) {
-        const int off0 = ((2 * lgrp) ^ f_sw) << 4;
-        const int off1 = ((2 * lgrp + 1) ^ f_sw) << 4;
+        // Lane group g feeds K slot [32 g, 32 g + 32) of the MFMA with bytes [16 g, 16 g + 16) and
+        // [64 + 16 g, 64 + 16 g + 16) of the step: activations and weights are permuted alike, so the
+        // sum is the same, and each of the two reads has the int8 kernels' conflict-free pattern (the
+        // four groups of a row read four neighbouring 16-byte pieces; reading pieces 2 g and 2 g + 1
+        // instead costs a two-way bank conflict on every read).
+        const int off0 = (lgrp ^ f_sw) << 4;
+        const int off1 = ((4 + lgrp) ^ f_sw) << 4;
         const uint8_t* src = (i < TM) ? As + buf * BM * BK + a_frag + i * 16 * BK : Bs + buf * BN * BK + b_frag + (i - TM) * 16 * BK;
         const v4i lo = *reinterpret_cast<const v4i*>(src + off0);
         const v4i hi = *reinterpret_cast<const v4i*>(src + off1);

@@ -11,7 +11,7 @@ moves to and from HBM come from two separate runs of the same command, one per c
         python3 REPO/bench.py --steps 5 --warmup 2 --ramp 3 --no-cpu --no-e4m3 --calib-copy [--config N]
     python3 -m segquant_amd.profile_counters OUT/fetch OUT/write --config N
 
-``--calib-copy`` makes bench.py launch one plain 256 MiB -> 256 MiB elementwise copy; what each
+``--calib-copy`` makes bench.py launch one plain 256 MiB -> 256 MiB elementwise pass (int32 times one); what each
 counter reads for that copy gives the counter's unit (the factor to KiB).  The result is merged
 into ``profiles/hbm_traffic.json`` under the configuration's number; bench.py copies it into its
 ``roofline`` object as ``traffic`` with ``traffic_source`` saying where it came from.
@@ -54,9 +54,10 @@ def main():
     launches = None
     for counter, path in (("FETCH_SIZE", args.fetch_dir), ("WRITE_SIZE", args.write_dir)):
         agg = _per_kernel(path, counter)
-        copy = [v for k, vs in agg.items() if "elementwise" in k and "copy" not in k.lower() for v in vs if v > 0.2 * COPY_KIB / 4]
-        if not copy:
-            raise SystemExit(f"{counter}: the yardstick copy is not in the trace (was bench.py run with --calib-copy?)")
+        # the yardstick is the only int32 multiply-by-a-scalar in the run
+        copy = [v for k, vs in agg.items() if "MulFunctor<int>" in k for v in vs]
+        if len(copy) != 1:
+            raise SystemExit(f"{counter}: expected one yardstick copy in the trace, found {len(copy)} (was bench.py run with --calib-copy?)")
         factor = COPY_KIB / max(copy)  # counter units -> KiB
         kern = {k: vs for k, vs in agg.items() if args.kernel in k}
         n = sum(len(vs) for vs in kern.values())
