@@ -168,7 +168,16 @@ def main():
         torch.mul(src, 1, out=dst)
         torch.cuda.synchronize()
         del src, dst
-    for i in range(args.ramp + args.warmup):
+    # untimed: ramp, then warm-up.  The first ramp steps are clocked on their own, so that the
+    # line also says what a step costs right after start-up
+    n_cold = min(10, args.ramp)
+    torch.cuda.synchronize()
+    t_c0 = time.perf_counter()
+    for i in range(n_cold):
+        step(i)
+    torch.cuda.synchronize()
+    cold_ms = (time.perf_counter() - t_c0) / n_cold * 1e3 if n_cold else None
+    for i in range(n_cold, args.ramp + args.warmup):
         step(i)
     torch.cuda.synchronize()
     # the timed region: exactly args.steps steps, nothing else on the stream
@@ -260,6 +269,7 @@ def main():
     out = {
         "metric": "seg-GEMM TOPS + % MFMA peak (FLUX shapes, M=4608); quantize kernel GB/s",
         "value": round(value, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ramp_steps": args.ramp,
+        "cold_start_ms_per_step": None if cold_ms is None else round(cold_ms, 4),
         "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8" if fmt == "int8" else "fp8_e4m3", "data": "synthetic",
         "config": {"workload": f"config {args.config}: " + ", ".join(f"{s.name} M{s.M} K{s.K} N{s.N} {s.kernel_type}" for s in specs),

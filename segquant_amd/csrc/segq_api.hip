@@ -363,7 +363,8 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     //    workspace, and the second to arrive adds the two, adds the bias and rounds.  Workspace:
     //    two tile-sized shares per tile, one word per tile in which the first to arrive leaves the
     //    launch's stamp (a per-process counter: no clearing between launches, and a fresh workspace
-    //    may hold anything).
+    //    may hold anything) and which the second clears (so that a captured graph, which replays
+    //    the launch with the stamp it was recorded with, works too).
     //  * More shares: each workgroup writes an fp32 partial result, a second kernel sums them in the
     //    order of the shares.  Workspace: the partial results.
     // Either way the parking slots of all those workgroups follow (int8 with several ranges).
@@ -481,7 +482,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         p.arrived = reinterpret_cast<unsigned int*>(static_cast<uint8_t*>(d->workspace) + tiles * 2 * c.bm * c.bn * 4);
         p.bsA = p.bsB = p.bsC = p.bsSx = p.bsSw = 0;  // blockIdx.y counts shares here, not problems
         static unsigned int g_stamp = 0x5e690000u;
-        p.stamp = __atomic_add_fetch(&g_stamp, 1u, __ATOMIC_RELAXED);
+        do p.stamp = __atomic_add_fetch(&g_stamp, 1u, __ATOMIC_RELAXED); while (p.stamp == 0u);  // 0 means "cleared"
         return i8 ? launch_gemm_i8(p, cfg, fold, 2, st) : launch_gemm_f8(p, cfg, fold, 2, st);
     }
     if (splits > 1) {

@@ -1137,6 +1137,9 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 // launch's stamp, or anything at all in a fresh workspace) reads as "nobody yet"
                 const unsigned before = __hip_atomic_exchange(p.arrived + tile_id, p.stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 *flag = before == p.stamp;
+                // the second one clears the word: a replay of this very launch (a captured graph keeps
+                // the stamp it was recorded with) must find "nobody yet" again
+                if (before == p.stamp) __hip_atomic_store(p.arrived + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             __syncthreads();
             if (!*flag) return;

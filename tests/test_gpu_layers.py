@@ -259,6 +259,43 @@ def test_repeated_forwards_reuse_descriptors_and_buffers(config, M):
         assert codes1.data_ptr() != codes2.data_ptr()
 
 
+@pytest.mark.parametrize("config,M", [(1, None), (2, None), (4, 2048), (5, 1024)])
+def test_layer_forward_replays_from_a_captured_graph(config, M):
+    """The layer's forward recorded into a HIP graph (the quantise and GEMM launches, the expansion
+    of int4 weights, the sum of K shares; config 2's fc2 is two K shares that meet inside the launch,
+    config 5 at 1024 tokens four shares and parked ranges) and replayed four times, with the input
+    rewritten, other eager launches and synchronisations between the replays: every replay must
+    equal the eager forward on the data then in the input buffer, bit for bit."""
+    from segquant_amd import workloads as W
+    for spec in W.config_linears(config, M=M):
+        layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+        gen = torch.Generator().manual_seed(17)
+        variants = [x.to(spec.x_dtype).to(DEV)] + [
+            (x * (torch.rand(x.shape[1], generator=gen) + 0.5)).to(spec.x_dtype).to(DEV) for _ in range(3)]
+        eager = [layer(v).clone() for v in variants]
+        static_in = variants[0].clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # buffers, workspaces and kernel attributes of this stream exist before the capture
+            for _ in range(2):
+                layer(static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_out = layer(static_in)
+        for i in (0, 1, 2, 3, 1):
+            static_in.copy_(variants[i])
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, eager[i]), (spec.name, i)
+            again = layer(variants[(i + 1) % 4])  # the program's own eager work between replays
+            torch.cuda.synchronize()
+            assert torch.equal(again, eager[(i + 1) % 4]), (spec.name, i)
+        del graph, layer
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("fmt", ["int8", "fpe4m3"])
 def test_forward_parts_writes_the_concatenation_as_codes(fmt):
     """Config 5's proj_out fed by its two producers (attention output, MLP output before its
