@@ -118,7 +118,8 @@ def e4m3_encode(v) -> np.ndarray:
     Restates the hardware cast the reference relies on,
     ``static_cast<__nv_fp8_e4m3>(float)`` (segquant/src/real_quant/quantizer.cuh:21-29,
     segquant/src/fake_quant/quantizer_fp8.cpp:35-36).  The sign of a NaN is
-    dropped (0x7F), which is the value the reference's survey of that cast records.
+    dropped (0x7F): what CUDA's conversion is documented to return for a NaN input (no run of
+    it was possible here, so this case is not pinned by a reference output).
     """
     v = _f32(v)
     shape = v.shape
