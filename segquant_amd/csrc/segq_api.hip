@@ -66,7 +66,9 @@ static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
     };
-    if (wide_ok && tiles(FIRST_WIDE_CFG + 3) >= 96) {
+    // (plain 8-bit operands go to the 8-wave kernels from 32 tiles of 128 x 128 up: 64 x 9216 x 3072 runs
+    // 24.9 us there against 35.2 us on the general kernel)
+    if (wide_ok && tiles(FIRST_WIDE_CFG + 3) >= (plain8 && !fold ? 32 : 96)) {
         // Short contractions of middling size: the plain 128 x 128 kernel needs ~100 registers, so two
         // workgroups share a CU and each one's prologue and epilogue (most of a tile's time at a dozen
         // K steps) run under the other's MFMAs.  Measured at K = 1280 .. 1536: 2048 x 10240 34.5 vs 45.5 us
@@ -385,7 +387,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
             if (d->split_k > 1) {
                 want = (int)(d->split_k < total_steps ? d->split_k : total_steps);
                 if (d->tile == 0) scfg = big_ok ? FIRST_WIDE_CFG : FIRST_WIDE_CFG + 1;
-            } else if (d->tile == 0 && total_steps >= 32 && tiles_of(cfg) * 10 < cus * 9) {
+            } else if (d->tile == 0 && total_steps >= 16 && tiles_of(cfg) * 10 < cus * 9) {
                 // Whole tiles would leave more than a tenth of the CUs idle: look for a big tile and a
                 // number of shares that fill them.  Measured (us, random codes, 256 CUs):
                 //   1024 x 3072, K 13824 twice (DualScale):  e4m3  256x192 x4 99 | 256x256 x5 130 | 128x128 176
@@ -403,10 +405,13 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
                     return (double)((wgs + cus - 1) / cus) * ((double)total_steps / s_ + 6.0 + (s_ > 1 ? 8.0 : 0.0)) *
                            TILE_CFGS[c].bm * TILE_CFGS[c].bn / eff(c);
                 };
-                const int cands[3] = {FIRST_WIDE_CFG + 6, FIRST_WIDE_CFG, FIRST_WIDE_CFG + 7};
+                // (the 128 x 128 tile joins for very few tokens: 64 x 9216 x 3072 in two or three shares
+                // 19 us against 25 us whole)
+                const int cands[4] = {FIRST_WIDE_CFG + 6, FIRST_WIDE_CFG, FIRST_WIDE_CFG + 7, FIRST_WIDE_CFG + 3};
                 double best = cost(cfg, 1);
-                for (int i = 0; i < (big_ok ? 3 : 1); ++i) {
+                for (int i = 0; i < (big_ok ? 4 : 1); ++i) {
                     const int c = big_ok ? cands[i] : FIRST_WIDE_CFG + 1;
+                    if (c == FIRST_WIDE_CFG + 3 && (d->m > 128 || (i8 && fold))) continue;
                     int64_t s_ = cus / tiles_of(c);
                     if (s_ > total_steps / 8) s_ = total_steps / 8;
                     if (s_ > 16) s_ = 16;
