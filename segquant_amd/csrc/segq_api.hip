@@ -350,6 +350,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;
     else return fail(SEGQ_ERR_ARG, "segq_gemm: tile %d is not in 0..%d", d->tile, NUM_TILE_CFG);
+    // Few tokens: when the 128 x 128 tiles do not even fill the CUs once, a workgroup has its CU to
+    // itself and waits on HBM latency: the int8 kernel with four LDS stages keeps three K steps in
+    // flight instead of one (256 x 9216 x 1536: 14.8 -> 12.9 us, 512 x 6144 x 3072: 25.5 -> 20.4 us)
+    if (d->tile == 0 && cfg == FIRST_WIDE_CFG + 3 && i8 && plain8 && !fold && !groups && !lowrank && wide_ok &&
+        ((d->m + 127) / 128) * ((d->n + 127) / 128) * d->batch <= device_cus() && ktotal / 128 >= 6)
+        cfg = FIRST_WIDE_CFG + 8;
     // the 8-wave tiles that exist with the finish in output units (low-rank branch, two-way K split)
     auto tail_tile = [](int c) {
         const int w = c - FIRST_WIDE_CFG;

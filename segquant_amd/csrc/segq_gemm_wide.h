@@ -1250,6 +1250,12 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 5: SEGQ_PIPE1(288, 192, 2, 4, false, false);
                     case 6: SEGQ_PIPE2(256, 192, 4, 2, false, false);
                     case 7: SEGQ_PIPE2(192, 256, 2, 4, false, false);
+                    case 8:  // four LDS stages: three K steps in flight per CU, for shapes that wait on HBM latency
+                        if constexpr (!F8W) {
+                            if (tail) break;
+                            return launch_pipe_instance<128, 128, 2, 4, FMT, false, 4, false, false, false>(p, batch, st);
+                        }
+                        break;
                 }
             } else if constexpr (F8W) {  // fp32 accumulators are rescaled in place: every tile serves several ranges
                 switch (wcfg) {

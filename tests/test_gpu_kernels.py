@@ -289,6 +289,40 @@ def test_gemm_eight_wave_tiles(ops, tile, fa, fb, M, N, K):
     assert (np.abs(got2 - want2) <= 4e-6 * (np.abs(p0) + np.abs(p1) + np.abs(bias.numpy())[None, :]) + slack2).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 2176, 1536), (200, 330, 128), (77, 130, 256), (130, 260, 384), (64, 1152, 768)])
+def test_gemm_four_stage_kernel_for_few_tokens(ops, M, N, K):
+    """Tile 19: the int8 128 x 128 kernel with four LDS stages (the library's own choice when the
+    tiles do not fill the CUs once).  Contractions shorter than, equal to and longer than the
+    number of stages, ragged M and N: raw accumulators exact, the fused fp32 and bf16 epilogues
+    within their rounding of the closed form; what it does not serve is refused."""
+    fmt = O.FMT_INT8
+    a, b = _rand_codes((M, K), fmt, 81), _rand_codes((N, K), fmt, 82)
+    ad, bd = _to_dev_codes(a, fmt), _to_dev_codes(b, fmt)
+    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, tile=19)
+    ref = O.gemm_acc(a, b, fmt, fmt)
+    out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+    assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
+    g = torch.Generator().manual_seed(83)
+    sx, sw, bias = torch.rand(M, generator=g) + 0.5, torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    want = ref / (sx.numpy().astype(np.float64)[:, None] * sw.numpy().astype(np.float64)[None, :]) + bias.numpy()
+    rg = [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
+    y32 = ops.gemm(ad, bd, rg, out_dtype=torch.float32, bias=bias.to(DEV), **kw)
+    assert np.abs(_np(y32).astype(np.float64) - want).max() <= 2e-6 * np.abs(want).max()
+    y16 = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **kw)
+    assert (np.abs(y16.float().cpu().numpy().astype(np.float64) - want) <= _bf16_ulp(want)).all()
+    if -(-M // 128) * -(-N // 128) >= 32:  # the library's own choice for such a shape
+        gd = ops.gemm_desc(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **{**kw, "tile": 0})
+        assert ops.gemm_plan(gd)["tile"] == 19
+        assert torch.equal(ops.gemm_launch(gd, None), y16)
+    two = [ops.Range(0, 128, sx.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(128, K - 128, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
+    if K > 128:
+        with pytest.raises(RuntimeError):  # one range only
+            ops.gemm(ad, bd, two, out_dtype=torch.float32, **kw)
+    e_a, e_b = _to_dev_codes(_rand_codes((M, K), O.FMT_E4M3, 84), O.FMT_E4M3), _to_dev_codes(_rand_codes((N, K), O.FMT_E4M3, 85), O.FMT_E4M3)
+    with pytest.raises(RuntimeError):  # int8 only
+        ops.gemm(e_a, e_b, [ops.Range(0, K, None, None)], out_dtype="acc", **{**kw, "a_fmt": O.FMT_E4M3, "b_fmt": O.FMT_E4M3})
+
+
 @pytest.mark.parametrize("tile", [0, 11, 15, 16])
 def test_gemm_more_tiles_than_compute_units(ops, tile):
     """4608 x 4608 outputs are 324 to 384 tiles, more than the 256 CUs hold at once."""
