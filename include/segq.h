@@ -257,11 +257,13 @@ typedef struct segq_gemm_desc {
     int64_t ld_addend;
     int64_t split_k;    /* 0: the library decides; 1: never; s > 1: the K steps of every tile are shared by s
                          * workgroups.  Splitting needs plain int8 or e4m3 codes, K ranges in multiples of 128,
-                         * batch == 1 and s * m * n * 4 bytes of workspace for the fp32 partial results (plus s
-                         * times the parking room above for int8 with several ranges); a second small kernel
-                         * sums them, adds the bias and rounds once.  For shapes with far fewer tiles than
-                         * compute units; no counterpart in the reference (its GemmUniversal runs one K
-                         * slice per problem: mode kGemm with batch_count 1,
+                         * batch == 1 and a workspace (segq_gemm_workspace_bytes says how much: the fp32 shares,
+                         * plus the parking room above per share for int8 with several ranges).  Two shares
+                         * meet inside the launch: the second workgroup to arrive at a tile adds the other's
+                         * share to its own, adds the bias and rounds (a + b = b + a: the same bits whoever is
+                         * last).  More shares are summed in their order by a second small kernel.  For shapes
+                         * whose whole tiles would leave compute units idle; no counterpart in the reference
+                         * (its GemmUniversal runs one K slice per problem: mode kGemm with batch_count 1,
                          * segquant/src/real_quant/real_gemm.cu:281-285 and :424-445). */
     const void* lowrank_t;  /* device or NULL.  A low-rank branch added to the result before its one rounding:
                          *   out[m][n] += sum_{k < lowrank_rank} lowrank_t[m][k] * lowrank_l2t[n][k]
