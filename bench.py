@@ -19,12 +19,12 @@ if ROOT not in sys.path:
 
 PEAK_TOPS = {"int8": 5000.0, "fpe4m3": 5000.0}  # dense MFMA, TOP/s
 PEAK_HBM = 8000.0                               # GB/s
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_configs_1_to_5.txt")
 
 
 def recorded_traffic(config):
     """HBM-side bytes per GEMM launch from the last rocprofv3 counter runs of this workload
-    (counters cannot be read from inside this process): profiles/hbm_traffic.json, written by
+    (counters cannot be read from inside this process): profiles/gemm_hbm_traffic_configs_1_to_5.txt, written by
     `python -m segquant_amd.profile_counters`.  (bytes or None, where the figure comes from)."""
     try:
         rec = json.load(open(TRAFFIC_FILE)).get(str(config))
@@ -32,7 +32,7 @@ def recorded_traffic(config):
         rec = None
     if not rec:
         return None, "no counter run recorded for this workload"
-    return rec["traffic_bytes_per_launch"], f"profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {rec.get('commit', '?')})"
+    return rec["traffic_bytes_per_launch"], f"profiles/gemm_hbm_traffic_configs_1_to_5.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {rec.get('commit', '?')})"
 
 
 def cpu_baseline(specs, rows, repeats=5):

@@ -13,7 +13,7 @@ moves to and from HBM come from two separate runs of the same command, one per c
 
 ``--calib-copy`` makes bench.py launch one plain 256 MiB -> 256 MiB elementwise pass (int32 times one); what each
 counter reads for that copy gives the counter's unit (the factor to KiB).  The result is merged
-into ``profiles/hbm_traffic.json`` under the configuration's number; bench.py copies it into its
+into ``profiles/gemm_hbm_traffic_configs_1_to_5.txt`` under the configuration's number; bench.py copies it into its
 ``roofline`` object as ``traffic`` with ``traffic_source`` saying where it came from.
 """
 from __future__ import annotations
@@ -27,7 +27,7 @@ import os
 import subprocess
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-OUT = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+OUT = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_configs_1_to_5.txt")
 COPY_KIB = 256 * 1024  # the yardstick copy reads and writes this many KiB
 
 
