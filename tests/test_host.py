@@ -456,3 +456,70 @@ def test_smooth_and_svd_layers_on_the_fake_path_equal_the_oracle(opt_type, seg_m
     with pytest.raises(NotImplementedError):
         SegmentLinear(K, N, input_quant_type="int8", weight_quant_type="int8", opt_type=opt_type,
                       opt_kwargs={"search_alpha_config": {"enable": True, "min": 0.1, "max": 0.9, "step": 0.1}}, device="cpu")
+
+
+def _plan(lib, m, n, ranges, fmt, out_dtype=2, lend=True, split_k=0, tile=0, lowrank=0):
+    """segq_gemm_plan / segq_gemm_workspace_bytes on a descriptor of made-up (aligned, never
+    dereferenced) device addresses: the library's decisions are host arithmetic and launch nothing.
+    ranges: (k_begin, k_len, a_sel).  Returns (tile id, K shares, parked, workspace bytes)."""
+    import ctypes as C
+    from segquant_amd import _lib as L
+    d = L.GemmDesc()
+    d.a_fmt = d.b_fmt = fmt
+    d.out_dtype = d.bias_dtype = out_dtype  # 2: bf16
+    k = max(b + l for b, l, _ in ranges)
+    d.m, d.n, d.lda, d.ldb, d.ldo, d.batch = m, n, k, k, n, 1
+    d.a, d.a_neg, d.b, d.out, d.bias = 0x10000000, 0x20000000, 0x30000000, 0x40000000, 0x50000000
+    d.n_ranges, d.tile, d.split_k = len(ranges), tile, split_k
+    for i, (b, l, sel) in enumerate(ranges):
+        d.ranges[i].k_begin, d.ranges[i].k_len, d.ranges[i].a_sel = b, l, sel
+        d.ranges[i].sx_row_stride, d.ranges[i].sw_col_stride = 1, 1
+        d.ranges[i].sx, d.ranges[i].sw = 0x60000000, 0x70000000
+    if lowrank:
+        d.lowrank_t, d.lowrank_l2t, d.lowrank_rank, d.ld_lowrank_t, d.ld_lowrank_l2t = 0x80000000, 0x90000000, lowrank, lowrank, lowrank
+    need = C.c_int64(-1)
+    assert lib.segq_gemm_workspace_bytes(C.byref(d), C.byref(need)) == 0, lib.segq_last_error()
+    if lend:
+        d.workspace, d.workspace_bytes = 0xA0000000, max(need.value, 16)
+    t, s, p = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    assert lib.segq_gemm_plan(C.byref(d), C.byref(t), C.byref(s), C.byref(p)) == 0, lib.segq_last_error()
+    return t.value, s.value, p.value, need.value
+
+
+def test_tile_and_share_choice_for_the_benchmark_shapes():
+    """What the library picks (tile id, K shares, parking) for the shapes of the five benchmark
+    configurations and for a few-token shape, with a workspace of the size it asks for and without
+    one.  Pure host arithmetic: no GPU, nothing launched.  (256 CUs are assumed when there is no
+    device to ask.)"""
+    import ctypes as C
+    from segquant_amd import _lib as L
+    lib = L.lib()
+    lib.segq_last_error.restype = C.c_char_p
+    I8, F8 = 0, 1
+    one = lambda k: [(0, k, 0)]
+    c5 = [(0, 3072, 0), (3072, 12288, 0), (3072, 12288, 1)]   # attn | MLP positive codes | MLP negative codes
+    fc2 = [(0, 6144, 0), (0, 6144, 1)]
+    # configuration 3: whole rounds of 256 CUs with 192x288 / 288x192 tiles, nothing split
+    assert _plan(lib, 4608, 9216, one(3072), I8)[:3] == (15, 1, 0)
+    assert _plan(lib, 4608, 12288, one(3072), I8)[:3] == (16, 1, 0)
+    assert _plan(lib, 4608, 3072, one(12288), I8)[:3] == (16, 1, 0)
+    # configuration 1: 144 tiles of 128x128 do not fill the CUs: the four-stage kernel; fp32 output (0)
+    assert _plan(lib, 256, 9216, one(1536), I8, out_dtype=0)[:3] == (19, 1, 0)
+    # configuration 2: fc1 in two whole rounds of 256x192; fc2 (DualScale: two ranges) as 128 tiles in two K shares
+    assert _plan(lib, 4096, 6144, one(1536), F8)[:3] == (17, 1, 0)
+    t, s, p, need = _plan(lib, 4096, 1536, fc2, F8)
+    assert (t, s, p) == (17, 2, 0) and need == 128 * 2 * 256 * 192 * 4 + 128 * 4 + (-(128 * 4) % 256)
+    assert _plan(lib, 4096, 1536, fc2, F8, lend=False)[1] == 1          # no workspace: no shares
+    assert _plan(lib, 4096, 1536, fc2, F8, split_k=1)[1] == 1           # forbidden by the caller
+    # configuration 5: 1024 tokens in 64 tiles x 4 shares (int8: parked ranges too), 4608 and 9216 whole
+    assert _plan(lib, 1024, 3072, c5, F8)[:3] == (17, 4, 0)
+    assert _plan(lib, 1024, 3072, c5, I8)[:3] == (17, 4, 1)
+    assert _plan(lib, 4608, 3072, c5, I8)[:3] == (16, 1, 1)
+    assert _plan(lib, 9216, 3072, c5, F8)[:3] == (16, 1, 0)
+    t, s, p, need = _plan(lib, 4608, 3072, c5, I8, lend=False)          # int8, several ranges, nothing lent:
+    assert p == 0 and need == 256 * 288 * 192 * 4 and t in (12, 13, 14)  # a second register set, smaller tiles
+    # few tokens: K shares of the 128x128 tile
+    t, s, p, _ = _plan(lib, 64, 9216, one(3072), I8)
+    assert t == 14 and s in (2, 3)
+    # the low-rank branch moves to a tile that is built with it
+    assert _plan(lib, 4608, 12288, one(3072), I8, lowrank=32)[:2] == (11, 1)
