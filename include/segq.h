@@ -137,6 +137,15 @@ typedef struct segq_quant_desc {
 
 int segq_quantize(const segq_quant_desc* d, segq_stream_t stream);
 
+/* n descriptors in order, with the results of n segq_quantize calls.  Neighbouring descriptors
+ * that one kernel instance serves (dynamic per-row scales, one column segment, no pre_op or
+ * col_div, 16-bit input, int8 or e4m3 codes, rows of up to 8192 elements in the same length class,
+ * the same `dual`) share one launch, up to four at a time: launches of a few tens of MB are a third
+ * ramp and tail.  For inputs that exist at the same time (the image and text streams of a
+ * double-stream block, whose projections the reference quantises one tensor at a time,
+ * segquant/src/real_quant/real_gemm.cu:700-716).  The outputs must not overlap. */
+int segq_quantize_many(const segq_quant_desc* descs, int32_t n, segq_stream_t stream);
+
 /* The reference's two weight entry points under their own names
  * (segquant/src/real_quant/seg_utils.h:82-119): one scale by value, or one per
  * output row.  weights is (n, k) row-major contiguous; codes is (n, k) bytes,

@@ -64,7 +64,7 @@ class GemmDesc(C.Structure):
 
 
 EXPORTS = (
-    "segq_version", "segq_last_error", "segq_quantize", "segq_quantize_weights_scalar",
+    "segq_version", "segq_last_error", "segq_quantize", "segq_quantize_many", "segq_quantize_weights_scalar",
     "segq_quantize_weights_rows", "segq_quantize_weights_groups", "segq_repack_int4_cols_to_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3",
     "segq_gemm_noalloc", "segq_noalloc_scratch_bytes", "segq_init",
 )
@@ -100,6 +100,7 @@ def lib() -> C.CDLL:
     L.segq_version.restype = C.c_int
     L.segq_last_error.restype = C.c_char_p
     L.segq_quantize.argtypes = [C.POINTER(QuantDesc), C.c_void_p]
+    L.segq_quantize_many.argtypes = [C.POINTER(QuantDesc), C.c_int32, C.c_void_p]
     L.segq_quantize_weights_scalar.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p,
                                                C.c_int32, C.c_float, C.c_void_p]
     L.segq_quantize_weights_rows.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p,

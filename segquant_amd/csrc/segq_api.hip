@@ -46,6 +46,7 @@ int reserve_lds(const void* kern, int bytes, unsigned long long* done) {
 }
 
 int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value);
+int quantize_many_impl(const segq_quant_desc* descs, int32_t n, hipStream_t st);
 int fake_e4m3_impl(const void* x, void* out, int32_t dtype, int64_t numel, hipStream_t st);
 int quantize_groups_impl(const void* w, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t fmt, const float* scales,
                          int64_t group, hipStream_t st);
@@ -567,6 +568,10 @@ const char* segq_last_error(void) { return g_err; }
 
 int segq_quantize(const segq_quant_desc* d, segq_stream_t stream) {
     return quantize_impl(d, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int segq_quantize_many(const segq_quant_desc* descs, int32_t n, segq_stream_t stream) {
+    return quantize_many_impl(descs, n, static_cast<hipStream_t>(stream));
 }
 
 static void weight_desc(segq_quant_desc* q, const void* w, int32_t w_dtype, int64_t n, int64_t k, void* codes, int32_t fmt) {

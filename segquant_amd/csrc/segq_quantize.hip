@@ -493,9 +493,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
 // 9216 x 3072 19.7 -> 17.7 us, 8192 x 1280 11.0 -> 9.1 us.  (A version whose waves
 // walked several rows with the next row's loads in flight measured the same.)
 template <int DT, int FMT, int CPL, bool DUAL>
-__global__ void __launch_bounds__(64) quant_dynamic_row_kernel(const QuantParams p) {
-    const int lane = threadIdx.x;
-    const int64_t row = blockIdx.x;
+__device__ __forceinline__ void quant_dynamic_row_body(const QuantParams& p, const int64_t row, const int lane) {
     const size_t esz = (DT == SEGQ_F32) ? 4 : 2;
     const int c1 = (int)(p.cols >> 4);
     const float eps = 5.9604644775390625e-08f;  // 2^-24
@@ -540,6 +538,27 @@ __global__ void __launch_bounds__(64) quant_dynamic_row_kernel(const QuantParams
             }
         }
     }
+}
+
+template <int DT, int FMT, int CPL, bool DUAL>
+__global__ void __launch_bounds__(64) quant_dynamic_row_kernel(const QuantParams p) {
+    quant_dynamic_row_body<DT, FMT, CPL, DUAL>(p, blockIdx.x, threadIdx.x);
+}
+
+// The same for up to SEGQ_QUANT_BATCH tensors in one grid: workgroup w serves row w - first[i] of tensor i.
+constexpr int SEGQ_QUANT_BATCH = 4;
+struct QuantBatch {
+    int32_t n;
+    int32_t first[SEGQ_QUANT_BATCH + 1];  // first workgroup of each tensor, then the grid size
+    QuantParams p[SEGQ_QUANT_BATCH];
+};
+
+template <int DT, int FMT, int CPL, bool DUAL>
+__global__ void __launch_bounds__(64) quant_dynamic_row_many_kernel(const QuantBatch b) {
+    const int w = blockIdx.x;
+    int i = 0;
+    while (i + 1 < b.n && w >= b.first[i + 1]) ++i;
+    quant_dynamic_row_body<DT, FMT, CPL, DUAL>(b.p[i], w - b.first[i], threadIdx.x);
 }
 
 
@@ -645,10 +664,12 @@ static int launch_quant_fmt(const QuantParams& p, hipStream_t st) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value) {
+// Checks a descriptor and turns it into kernel parameters.  *empty: nothing to do (no rows or no columns).
+static int quant_params(const segq_quant_desc* d, const float* scale_by_value, QuantParams& p, bool* empty) {
+    *empty = false;
     if (!d) return fail(SEGQ_ERR_ARG, "segq_quantize: null descriptor");
     if (d->rows < 0 || d->cols < 0) return fail(SEGQ_ERR_ARG, "segq_quantize: negative size");
-    if (d->rows == 0 || d->cols == 0) return SEGQ_OK;
+    if (d->rows == 0 || d->cols == 0) { *empty = true; return SEGQ_OK; }
     if (!d->x || !d->codes || (!d->scale && !scale_by_value))
         return fail(SEGQ_ERR_ARG, "segq_quantize: null x, codes or scale");
     if (scale_by_value && (d->dual || d->dynamic))
@@ -669,7 +690,7 @@ int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_b
     if (d->rows * (d->cols / 16) > (int64_t)0x7fffffff * 256 || d->cols > 0x7fffffff || d->rows > 0x7fffffff)
         return fail(SEGQ_ERR_ARG, "segq_quantize: matrix too large");
 
-    QuantParams p{};
+    p = QuantParams{};
     p.x = d->x; p.codes = d->codes; p.codes_neg = d->codes_neg;
     p.scale = d->scale; p.scale_neg = d->scale_neg;
     p.rows = d->rows; p.cols = d->cols; p.ldx = d->ldx; p.ldc = d->ld_codes;
@@ -701,11 +722,93 @@ int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_b
     }
     if (p.dynamic && p.row_stride != 1 && p.rows != 1 && p.seg_rows != 1)
         return fail(SEGQ_ERR_ARG, "segq_quantize: dynamic scales are per row (row_stride must be 1)");
-    switch (d->x_dtype) {
+    return SEGQ_OK;
+}
+
+static int launch_params(const QuantParams& p, hipStream_t st) {
+    switch (p.x_dtype) {
         case SEGQ_F32: return launch_quant_fmt<SEGQ_F32>(p, st);
         case SEGQ_F16: return launch_quant_fmt<SEGQ_F16>(p, st);
         default: return launch_quant_fmt<SEGQ_BF16>(p, st);
     }
+}
+
+int quantize_impl(const segq_quant_desc* d, hipStream_t st, const float* scale_by_value) {
+    QuantParams p;
+    bool empty;
+    if (const int rc = quant_params(d, scale_by_value, p, &empty)) return rc;
+    return empty ? SEGQ_OK : launch_params(p, st);
+}
+
+// Several tensors in one launch.  Two or more descriptors that the one-wave-per-row kernel serves
+// in the same instance (dynamic scales, one column segment, no fused producer, 16-bit input, int8
+// or e4m3 codes, rows of the same length class, the same DualScale setting) share a grid: a launch
+// of a few tens of MB is a third ramp and tail, which they then pay once (two 4608 x 3072 bf16
+// tensors: 2 x 10.8 us apart, ~16.5 us together).  Anything else is launched one by one.
+template <int DT, int FMT, int CPL>
+static int launch_row_batch(const QuantBatch& b, bool dual, hipStream_t st) {
+    const dim3 grid((unsigned)b.first[b.n]), one_wave(64);
+    if (dual) hipLaunchKernelGGL((quant_dynamic_row_many_kernel<DT, FMT, CPL, true>), grid, one_wave, 0, st, b);
+    else hipLaunchKernelGGL((quant_dynamic_row_many_kernel<DT, FMT, CPL, false>), grid, one_wave, 0, st, b);
+    return check_launch("segq_quantize_many");
+}
+
+template <int DT, int FMT>
+static int launch_row_batch_cpl(const QuantBatch& b, int cpl, bool dual, hipStream_t st) {
+    switch (cpl) {
+        case 1: return launch_row_batch<DT, FMT, 1>(b, dual, st);
+        case 2: return launch_row_batch<DT, FMT, 2>(b, dual, st);
+        case 3: return launch_row_batch<DT, FMT, 3>(b, dual, st);
+        case 4: return launch_row_batch<DT, FMT, 4>(b, dual, st);
+        case 6: return launch_row_batch<DT, FMT, 6>(b, dual, st);
+        default: return launch_row_batch<DT, FMT, 8>(b, dual, st);
+    }
+}
+
+static int row_cpl(const QuantParams& p) {  // runs of 16 per lane in the row kernel; 0: not its case
+    const int64_t runs = p.cols / 16;
+    if (!p.dynamic || p.n_kseg != 1 || p.pre_op || p.col_div || p.group || runs > 64 * 8) return 0;
+    if (p.x_dtype == SEGQ_F32 || (p.fmt != SEGQ_CODE_I8 && p.fmt != SEGQ_CODE_E4M3)) return 0;
+    if (p.dual && !(p.dual_mask & 1u)) return 0;
+    return runs <= 64 ? 1 : runs <= 128 ? 2 : runs <= 192 ? 3 : runs <= 256 ? 4 : runs <= 384 ? 6 : 8;
+}
+
+int quantize_many_impl(const segq_quant_desc* descs, int32_t n, hipStream_t st) {
+    if (n < 0 || (n > 0 && !descs)) return fail(SEGQ_ERR_ARG, "segq_quantize_many: bad descriptor array");
+    int i = 0;
+    while (i < n) {
+        QuantBatch b{};
+        bool empty;
+        if (const int rc = quant_params(&descs[i], nullptr, b.p[0], &empty)) return rc;
+        if (empty) { ++i; continue; }
+        const int cpl = row_cpl(b.p[0]);
+        b.n = 1;
+        b.first[0] = 0; b.first[1] = (int32_t)b.p[0].rows;
+        int j = i + 1;
+        while (cpl && j < n && b.n < SEGQ_QUANT_BATCH) {  // gather the descriptors that follow and fit the same instance
+            QuantParams q;
+            if (const int rc = quant_params(&descs[j], nullptr, q, &empty)) return rc;
+            if (empty || row_cpl(q) != cpl || q.x_dtype != b.p[0].x_dtype || q.fmt != b.p[0].fmt || q.dual != b.p[0].dual ||
+                (int64_t)b.first[b.n] + q.rows > 0x7fffffff)
+                break;
+            b.p[b.n] = q;
+            b.first[b.n + 1] = b.first[b.n] + (int32_t)q.rows;
+            ++b.n; ++j;
+        }
+        int rc;
+        if (b.n == 1) {
+            rc = launch_params(b.p[0], st);
+        } else {
+            const bool dual = b.p[0].dual != 0, f8 = b.p[0].fmt == SEGQ_CODE_E4M3;
+            if (b.p[0].x_dtype == SEGQ_BF16)
+                rc = f8 ? launch_row_batch_cpl<SEGQ_BF16, SEGQ_CODE_E4M3>(b, cpl, dual, st) : launch_row_batch_cpl<SEGQ_BF16, SEGQ_CODE_I8>(b, cpl, dual, st);
+            else
+                rc = f8 ? launch_row_batch_cpl<SEGQ_F16, SEGQ_CODE_E4M3>(b, cpl, dual, st) : launch_row_batch_cpl<SEGQ_F16, SEGQ_CODE_I8>(b, cpl, dual, st);
+        }
+        if (rc) return rc;
+        i = j;
+    }
+    return SEGQ_OK;
 }
 
 // Weight codes with one scale per (row, group of `group` contraction columns): the static kernel

@@ -131,6 +131,18 @@ def quantize_launch(q):
     return result
 
 
+def quantize_many(qs):
+    """Enqueue several quantise launches (tuples from :func:`quantize_desc`) through one
+    ``segq_quantize_many`` call: neighbours that the same kernel instance serves share a launch.
+    Returns the code tensor(s) of each."""
+    if not qs:
+        return []
+    arr = (L.QuantDesc * len(qs))(*[q[0] for q in qs])  # (copies of the descriptors; the tensors stay alive in qs)
+    info = dict(many=[q[2] for q in qs])
+    L.check(_launch("quantize", info, lambda: L.lib().segq_quantize_many(arr, len(qs), _stream())))
+    return [q[1] for q in qs]
+
+
 def quantize_desc(x: torch.Tensor, fmt: str, scale: torch.Tensor, scale_neg: Optional[torch.Tensor] = None, *,
              seg_rows: int = 0, seg_stride: int = 0, row_stride: int = 0,
              kseg_bounds: Optional[Sequence[int]] = None, kseg_stride: int = 0,

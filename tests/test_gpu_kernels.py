@@ -165,6 +165,53 @@ def test_quantize_dynamic_per_row(ops, fmt, dual):
     assert np.array_equal(_codes_np(c, fmt), want)
 
 
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("dual", [False, True])
+def test_quantize_many_shares_launches_and_matches_single_calls(ops, fmt, dual):
+    """segq_quantize_many: tensors of the same kind (dynamic per-row scales, one column segment,
+    the same row-length class) go through one launch, others through their own, in any mix and
+    order; codes and scales are those of one segq_quantize call each, bit for bit.  Five batchable
+    tensors in a row (more than one shared launch holds), a longer row class in between, an fp32
+    input, a static one and an empty one."""
+    g = torch.Generator().manual_seed(91)
+    def dyn(M, K, dt=torch.bfloat16):
+        x = (torch.randn(M, K, generator=g) * 3).to(dt).to(DEV)
+        mk = lambda: (torch.empty(M, device=DEV), torch.empty(M, device=DEV) if dual else None)
+        return x, mk
+    cases = [dyn(37, 3072), dyn(5, 3056), dyn(64, 3072), dyn(129, 2960), dyn(3, 3072),   # one length class (CPL 3)
+             dyn(20, 5120), dyn(7, 3072), dyn(9, 3072, torch.float32), dyn(0, 3072), dyn(11, 3072, torch.float16),
+             dyn(4, 3072, torch.float16)]
+    single, many, keep = [], [], []
+    for x, mk in cases:
+        s1, n1 = mk()
+        single.append((ops.quantize(x, fmt, s1, n1, row_stride=1, dual=dual, dynamic=True) if x.shape[0] else None, s1, n1))
+        s2, n2 = mk()
+        if x.shape[0]:
+            many.append(ops.quantize_desc(x, fmt, s2, n2, row_stride=1, dual=dual, dynamic=True))
+        keep.append((s2, n2))
+    # a static per-tensor launch in the middle of the list
+    xs = (torch.randn(33, 3072, generator=g)).to(torch.bfloat16).to(DEV)
+    st = torch.full((1,), 17.5, device=DEV)
+    want_static = ops.quantize(xs, fmt, st)
+    many.insert(3, ops.quantize_desc(xs, fmt, st))
+    with ops.record_launches() as log:
+        res = ops.quantize_many(many)
+        torch.cuda.synchronize()
+    assert len(log) == 1  # one call into the library
+    got_static = res.pop(3)
+    assert torch.equal(got_static if not isinstance(got_static, tuple) else got_static[0],
+                       want_static if not isinstance(want_static, tuple) else want_static[0])
+    it = iter(res)
+    for (x, _), (c1, s1, n1), (s2, n2) in zip(cases, single, keep):
+        if not x.shape[0]:
+            continue
+        c2 = next(it)
+        assert torch.equal(s1, s2) and (n1 is None or torch.equal(n1, n2))
+        a, b = (c1 if isinstance(c1, tuple) else (c1,)), (c2 if isinstance(c2, tuple) else (c2,))
+        for u, v in zip(a, b):
+            assert torch.equal(u, v)
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 def test_quantize_weights_both_overloads(ops, fmt):
     N, K = 24, 64
