@@ -660,6 +660,7 @@ int segq_gemm_noalloc(const segq_gemm_desc* d, segq_stream_t stream) {
 
 int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream) {
     if (!q || !g) return fail(SEGQ_ERR_ARG, "segq_linear: null descriptor");
+    if (q->rows == 0 && g->m == 0) return SEGQ_OK;  // no token rows: nothing to quantise, nothing to multiply
     // the GEMM must consume exactly what the quantise step produces
     if (q->codes != g->a) return fail(SEGQ_ERR_ARG, "segq_linear: the GEMM must read the codes the quantise step writes");
     if (g->n_ranges < 1 || g->n_ranges > SEGQ_MAX_RANGES) return fail(SEGQ_ERR_ARG, "segq_linear: n_ranges %d out of range", g->n_ranges);

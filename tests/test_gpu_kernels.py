@@ -186,8 +186,7 @@ def test_quantize_many_shares_launches_and_matches_single_calls(ops, fmt, dual):
         s1, n1 = mk()
         single.append((ops.quantize(x, fmt, s1, n1, row_stride=1, dual=dual, dynamic=True) if x.shape[0] else None, s1, n1))
         s2, n2 = mk()
-        if x.shape[0]:
-            many.append(ops.quantize_desc(x, fmt, s2, n2, row_stride=1, dual=dual, dynamic=True))
+        many.append(ops.quantize_desc(x, fmt, s2, n2, row_stride=1, dual=dual, dynamic=True))
         keep.append((s2, n2))
     # a static per-tensor launch in the middle of the list
     xs = (torch.randn(33, 3072, generator=g)).to(torch.bfloat16).to(DEV)
@@ -203,9 +202,10 @@ def test_quantize_many_shares_launches_and_matches_single_calls(ops, fmt, dual):
                        want_static if not isinstance(want_static, tuple) else want_static[0])
     it = iter(res)
     for (x, _), (c1, s1, n1), (s2, n2) in zip(cases, single, keep):
-        if not x.shape[0]:
-            continue
         c2 = next(it)
+        if not x.shape[0]:
+            assert (c2[0] if isinstance(c2, tuple) else c2).shape[0] == 0
+            continue
         assert torch.equal(s1, s2) and (n1 is None or torch.equal(n1, n2))
         a, b = (c1 if isinstance(c1, tuple) else (c1,)), (c2 if isinstance(c2, tuple) else (c2,))
         for u, v in zip(a, b):
@@ -1110,3 +1110,29 @@ def test_gemm_low_rank_branch_in_the_epilogue(ops, fmt, dt, ranges, lend):
     with pytest.raises(RuntimeError, match="low-rank"):
         ops.gemm(ad, bd, rg[:1], m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=TDT[dt], lda=K, ldb=K, tile=3,
                  lowrank=(t_lr.to(TDT[dt]), l2t.to(TDT[dt])))
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+def test_empty_inputs_through_the_wrappers(ops, fmt):
+    """No rows to quantise, no rows or no columns to multiply: the calls succeed, give tensors of
+    the right empty shape and leave a poisoned neighbour untouched."""
+    K, N = 256, 192
+    x = torch.randn(0, K, dtype=torch.bfloat16, device=DEV)
+    s = torch.full((1,), 3.0, device=DEV)
+    codes = ops.quantize(x, fmt, s)
+    assert codes.shape == (0, K)
+    sd = torch.empty(0, device=DEV)
+    codes = ops.quantize(x, fmt, sd, row_stride=1, dynamic=True)
+    assert codes.shape == (0, K)
+    b = _to_dev_codes(_rand_codes((N, K), fmt, 5), fmt)
+    one = torch.ones(1, device=DEV)
+    guard = torch.full((4, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = ops.gemm(codes, b, [ops.Range(0, K, one, one, 0, 0, 0)], m=0, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.bfloat16,
+                   lda=K, ldb=K, out=guard[:0])
+    assert out.shape == (0, N)
+    a = _to_dev_codes(_rand_codes((8, K), fmt, 6), fmt)
+    out = ops.gemm(a, b[:0], [ops.Range(0, K, one, one, 0, 0, 0)], m=8, n=0, a_fmt=fmt, b_fmt=fmt, out_dtype=torch.bfloat16,
+                   lda=K, ldb=K)
+    assert out.shape == (8, 0)
+    torch.cuda.synchronize()
+    assert bool((guard == 7.0).all())

@@ -389,3 +389,21 @@ def test_smooth_layer_with_output_segments_takes_the_reference_route():
     out = layer(xd)
     ref = torch.nn.functional.linear(x.to(DEV), w.to(DEV), b.to(DEV))
     assert out.shape == (M, N) and ((out - ref).norm() / ref.norm()).item() < 0.05
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_zero_tokens_give_an_empty_output(config):
+    """An input with no token rows: the layers return (0, N) in the input's dtype on both
+    routes without launching anything that reads memory; the next call with rows is unaffected."""
+    from segquant_amd import workloads as W
+    spec = W.config_linears(config, M=64)[0]
+    layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+    xin = x.to(spec.x_dtype).to(DEV)
+    want = layer(xin).clone()
+    out = layer(xin[:0])
+    assert out.shape == (0, spec.N) and out.dtype == spec.x_dtype
+    if config not in (4, 5):  # (group-wise weight scales and unequal K segments run on the fused route only)
+        chunks = layer(xin[:0], chunked=True)
+        assert chunks.shape[-2] == 0
+    torch.cuda.synchronize()
+    assert torch.equal(layer(xin), want)

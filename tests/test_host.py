@@ -70,6 +70,34 @@ def test_argument_errors_are_reported_without_a_gpu():
         _lib.check(1)
 
 
+def test_empty_problems_succeed_before_any_device_work():
+    """No rows, no columns, no tensors in a list: nothing to launch, so the entry points return
+    SEGQ_OK without looking at pointers or the device; negative sizes are argument errors."""
+    from segquant_amd import _lib
+    lib = _lib.lib()
+    for m, n in ((0, 64), (64, 0), (0, 0)):
+        d = _lib.GemmDesc()
+        d.m, d.n, d.batch = m, n, 1
+        assert lib.segq_gemm(ctypes.byref(d), None) == 0
+    d = _lib.GemmDesc()
+    d.m, d.n, d.batch = -1, 4, 1
+    assert lib.segq_gemm(ctypes.byref(d), None) == 1
+    for rows, cols in ((0, 3072), (7, 0)):
+        q = _lib.QuantDesc()
+        q.rows, q.cols = rows, cols
+        assert lib.segq_quantize(ctypes.byref(q), None) == 0
+    q = _lib.QuantDesc()
+    q.rows, q.cols = -3, 16
+    assert lib.segq_quantize(ctypes.byref(q), None) == 1
+    assert lib.segq_quantize_many(None, 0, None) == 0
+    q, d = _lib.QuantDesc(), _lib.GemmDesc()
+    q.cols, q.dynamic, d.n, d.batch, d.n_ranges = 3072, 1, 64, 1, 1
+    assert lib.segq_linear(ctypes.byref(q), ctypes.byref(d), None) == 0
+    two = (_lib.QuantDesc * 2)()
+    two[0].rows, two[0].cols, two[1].rows, two[1].cols = 0, 3072, 5, 0
+    assert lib.segq_quantize_many(two, 2, None) == 0
+
+
 # ------------------------------------------------------------------ registry / loaders
 def test_ext_dict_has_the_reference_shape():
     from segquant_amd.layers import ext_dict
