@@ -313,25 +313,34 @@ __device__ __forceinline__ void load_run(const QuantParams& p, const uint8_t* xr
     if constexpr (PRE) pre_run<DT>(p, row, (int64_t)c << 4, r);
 }
 
-// Running maxima of the positive and of the negative side (strict masks x > 0 and
-// x < 0, segquant/quantizers/quantizer.py:172-189; NaN is ignored).  Without
-// DualScale only their maximum matters, which is one max of |x| per element.
+// Maximum of two non-negative floats, taken on their encodings: non-negative floats are ordered
+// like their bit patterns and every NaN pattern lies above infinity's, so a NaN wins and travels
+// on (fmaxf would drop it), as it does through torch's amax (segquant/quantizers/quantizer.py:212).
+__device__ __forceinline__ float max_nn(float a, float b) {
+    const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+    return __uint_as_float(ua > ub ? ua : ub);
+}
+
+// DualScale segments: running maxima of the positive and of the negative side (strict masks
+// x > 0 and x < 0, segquant/quantizers/quantizer.py:172-189; a NaN is on neither side).  Other
+// segments: the maximum of |x| in amax_p, NaN if the segment holds one.
 template <bool DUAL>
-__device__ __forceinline__ void track_amax(const float (&v)[16], float& amax_p, float& amax_n) {
+__device__ __forceinline__ void track_amax(const float (&v)[16], float& amax_p, float& amax_n, const bool dual = DUAL) {
+    if (DUAL && dual) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        if constexpr (DUAL) {
+        for (int j = 0; j < 16; ++j) {
             amax_p = fmaxf(amax_p, v[j]);    // starts at 0, so negatives never win
             amax_n = fmaxf(amax_n, -v[j]);
-        } else {
-            amax_p = fmaxf(amax_p, fabsf(v[j]));
         }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) amax_p = max_nn(amax_p, fabsf(v[j]));
     }
 }
 
-__device__ __forceinline__ float wave_max(float v) {
+__device__ __forceinline__ float wave_max(float v) {  // of non-negative values or NaN
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    for (int o = 32; o > 0; o >>= 1) v = max_nn(v, __shfl_xor(v, o, 64));
     return v;
 }
 
@@ -364,7 +373,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
             if (c < c1) {
                 float v[16];
                 raw_to_f32<DT>(raw[i], v);
-                track_amax<DUAL>(v, amax_p, amax_n);
+                track_amax<DUAL>(v, amax_p, amax_n, dual);
             }
         }
         for (int c = c0 + threadIdx.x + CACHE * 256; c < c1; c += 256) {
@@ -372,7 +381,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
             float v[16];
             load_run<DT, PRE>(p, xrow, row, c, t);
             raw_to_f32<DT>(t, v);
-            track_amax<DUAL>(v, amax_p, amax_n);
+            track_amax<DUAL>(v, amax_p, amax_n, dual);
         }
         amax_p = wave_max(amax_p);
         if constexpr (DUAL) amax_n = wave_max(amax_n);
@@ -382,14 +391,14 @@ __global__ void __launch_bounds__(256) quant_dynamic_kernel(const QuantParams p)
             red[1][threadIdx.x >> 6] = amax_n;
         }
         __syncthreads();
-        amax_p = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
-        amax_n = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+        amax_p = max_nn(max_nn(red[0][0], red[0][1]), max_nn(red[0][2], red[0][3]));
+        amax_n = max_nn(max_nn(red[1][0], red[1][1]), max_nn(red[1][2], red[1][3]));
         float s_pos, s_neg;
         if (dual) {
             s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
             s_neg = qmax_neg<FMT>() / fmaxf(amax_n, eps);
         } else {
-            s_pos = s_neg = qmax_pos<FMT>() / fmaxf(fmaxf(amax_p, amax_n), eps);
+            s_pos = s_neg = qmax_pos<FMT>() / max_nn(amax_p, eps);
         }
         const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
         if (threadIdx.x == 0) {
@@ -447,11 +456,11 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
             if (c < c1) {
                 if constexpr (KEEP) {
                     raw_to_f32<DT>(raw[i], vf[i]);
-                    track_amax<DUAL>(vf[i], amax_p, amax_n);
+                    track_amax<DUAL>(vf[i], amax_p, amax_n, dual);
                 } else {
                     float v[16];
                     raw_to_f32<DT>(raw[i], v);
-                    track_amax<DUAL>(v, amax_p, amax_n);
+                    track_amax<DUAL>(v, amax_p, amax_n, dual);
                 }
             }
         }
@@ -462,7 +471,7 @@ __global__ void __launch_bounds__(256) quant_dynamic_wave_kernel(const QuantPara
             s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
             s_neg = qmax_neg<FMT>() / fmaxf(amax_n, eps);
         } else {
-            s_pos = s_neg = qmax_pos<FMT>() / fmaxf(fmaxf(amax_p, amax_n), eps);
+            s_pos = s_neg = qmax_pos<FMT>() / max_nn(amax_p, eps);
         }
         const int64_t si = row_scale_index(p, row) + (int64_t)ks * p.kseg_stride;
         if (lane == 0) {
@@ -522,7 +531,7 @@ __device__ __forceinline__ void quant_dynamic_row_body(const QuantParams& p, con
             s_pos = qmax_pos<FMT>() / fmaxf(amax_p, eps);
             s_neg = qmax_neg<FMT>() / fmaxf(amax_n, eps);
         } else {
-            s_pos = s_neg = qmax_pos<FMT>() / fmaxf(amax_p, eps);
+            s_pos = s_neg = qmax_pos<FMT>() / max_nn(amax_p, eps);
         }
         const int64_t si = row_scale_index(p, row);
         if (lane == 0) {

@@ -167,6 +167,44 @@ def test_quantize_dynamic_per_row(ops, fmt, dual):
 
 @pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
 @pytest.mark.parametrize("dual", [False, True])
+@pytest.mark.parametrize("K", [3072, 4800, 12288])   # one wave per row and workgroup / per row / one workgroup per row
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_quantize_dynamic_rows_with_nan_inf_and_extremes(ops, fmt, dual, K, dt):
+    """Per-row scales of rows that hold a NaN, an infinity, a value next to the largest finite
+    one, or nothing above 1e-30.  A single scale is max|x| the way torch's amax takes it: a NaN
+    in the row makes the scale NaN and every code of the row the NaN code; DualScale's strict
+    masks leave a NaN on neither side (segquant/quantizers/quantizer.py:172-189, :212).  An
+    infinite maximum gives scale 0.  Scales and codes bit-exact against the oracle."""
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(7, K, generator=g)
+    x[1, 5] = float("nan"); x[2, 7] = float("inf"); x[3, 9] = float("-inf"); x[4, 11] = 3e38
+    x[5] = 0; x[5, 3] = 1e-30
+    x[6, K - 1] = float("nan")  # in the last lane's last run
+    x = x.to(TDT[dt]).to(DEV)
+    s = torch.empty(7, device=DEV)
+    sn = torch.empty(7, device=DEV) if dual else None
+    c = ops.quantize(x, fmt, s, sn, row_stride=1, dual=dual, dynamic=True)
+    xn = _np(x)
+    lim_p = {O.FMT_INT8: 127.0, O.FMT_E4M3: 448.0}[fmt]
+    lim_n = {O.FMT_INT8: 128.0, O.FMT_E4M3: 448.0}[fmt]
+    same = lambda a, b: np.array_equal(a, b, equal_nan=True)
+    with np.errstate(all="ignore"):
+        if dual:
+            pa, na = O.dual_amax(xn, axis=-1)
+            ws, wn = O.row_scale_div(pa, lim_p), O.row_scale_div(na, lim_n)
+            assert same(sn.cpu().numpy(), wn)
+            wp, wq = O.quantize_act_dual(xn[None], ws, wn, fmt)
+            want = O.merge_dual_codes(wp, wq, xn[None])[0]
+        else:
+            ws = O.row_scale_div(np.abs(xn).max(axis=-1), lim_p)
+            assert np.isnan(ws[1]) and np.isnan(ws[6]) and ws[2] == 0 and ws[3] == 0
+            want = O.quantize_act(xn[None], ws, fmt)[0]
+    assert same(s.cpu().numpy(), ws)
+    assert np.array_equal(_codes_np(c, fmt), want)
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("dual", [False, True])
 def test_quantize_many_shares_launches_and_matches_single_calls(ops, fmt, dual):
     """segq_quantize_many: tensors of the same kind (dynamic per-row scales, one column segment,
     the same row-length class) go through one launch, others through their own, in any mix and
