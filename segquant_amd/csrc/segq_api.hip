@@ -62,7 +62,8 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 // tiles of 256 x 256 beat 432 tiles of 256 x 128 by 30 %).  The 192 x 288 and
 // 288 x 192 tiles exist because 4608 rows of FLUX tokens make whole rounds with
 // them where 256 x 256 leaves the last round half empty.
-static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8, int64_t k_steps = 1 << 20) {  // fold: needs a second accumulator set
+static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide_ok, bool plain8, int64_t k_steps = 1 << 20,
+                       bool big_ok = false) {  // fold: needs a second accumulator set; big_ok: 384 x 192 serves this launch
     auto tiles = [&](int cfg) {
         const TileCfg& c = TILE_CFGS[cfg];
         return ((m + c.bm - 1) / c.bm) * ((n + c.bn - 1) / c.bn) * batch;
@@ -96,6 +97,16 @@ static int choose_tile(int64_t m, int64_t n, int64_t batch, bool fold, bool wide
                 best = cfg;
                 best_cost = cost;
             }
+        }
+        // 384 x 192, eight wave tiles of 96 x 96 (the fewest LDS bytes per MFMA of all tiles): taken when
+        // it tiles the output exactly, in whole rounds of the CUs, and with no more rounds x area than
+        // the choice above.  4608 x 12288 x 3072: three rounds instead of four of 288 x 192, e4m3 165 ->
+        // 140 us; 8192^3, which it does not tile exactly, is 12 % slower on it than on 256 x 256
+        const int big = FIRST_WIDE_CFG + 9;
+        if (big_ok && plain8 && !fold && batch == 1 && m % TILE_CFGS[big].bm == 0 && n % TILE_CFGS[big].bn == 0 && tiles(big) % cus == 0) {
+            const TileCfg& t = TILE_CFGS[best];
+            const int64_t rounds = (tiles(best) + cus - 1) / cus;
+            if (tiles(big) / cus * TILE_CFGS[big].bm * TILE_CFGS[big].bn <= rounds * t.bm * t.bn) return big;
         }
         return best;
     }
@@ -351,7 +362,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         } else {
             cfg = park ? choose_tile(d->m, d->n, d->batch, false, wide_ok, plain8) : -1;
             park = park && park_fits(cfg);
-            if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8, ktotal / 128);
+            if (!park) cfg = choose_tile(d->m, d->n, d->batch, fold2, wide_ok, plain8, ktotal / 128, (!fold || f8) && !lowrank);
         }
     }
     else if (d->tile >= 1 && d->tile <= NUM_TILE_CFG) cfg = d->tile - 1;

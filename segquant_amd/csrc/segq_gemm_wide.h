@@ -543,7 +543,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // which are converted at once, so no int32 accumulator set lives across
     // steps and the 64 x 64 wave tile fits.
     static_assert(!GRP || (!F8 && NS == 2), "group factors: int8, two stages");
-    constexpr bool S8 = F8 || GRP;  // whole-step fragments
+    // int8 tiles above 256 x 256 run the whole-step schedule too: one set of 32-byte fragments
+    // instead of two sets of 16-byte ones leaves room for their accumulators
+    constexpr bool WS = !F8 && !GRP && BM * BN > 256 * 256;
+    constexpr bool S8 = F8 || GRP || WS;  // whole-step fragments
     //
     // PARK (int8, several ranges): no second register set at all.  When a range
     // ends, its int32 sums are converted to the LAST range's units
@@ -554,6 +557,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // segments or DualScale: a few hundred KB of traffic per tile and range
     // boundary against ~14 MB of operands.
     static_assert(!PARK || (FOLD && !F8 && !GRP), "parking: int8 with several ranges");
+    static_assert(!WS || (!FOLD && !PARK), "int8 above 256 x 256: one range");
     constexpr bool ACCF = FOLD && !F8 && !GRP && !PARK;
     constexpr bool HASF = ACCF || GRP;
     const acc_t acc_zero = {0, 0, 0, 0};
@@ -938,6 +942,20 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 }
 #pragma unroll
                 for (int b = 0; b < TM; ++b) accf[a][b] += __builtin_convertvector(t[b], v4f) * g;
+            } else if constexpr (WS) {
+                // int8: the two 64-byte K halves of a block, TM MFMAs apart
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if (b == 0 && a == 0) frag8(buf, TM + 1);
+                    if (b == (TM > 1 ? 1 : 0)) frag8(buf, TM + a + 2);
+                    if constexpr (!F8) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo4(fb8[a]), lo4(fa8[b]), acc[a][b], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if constexpr (!F8) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi4(fb8[a]), hi4(fa8[b]), acc[a][b], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             } else {
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
@@ -980,6 +998,26 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
                 }
 #pragma unroll
                 for (int b = 0; b < TM; ++b) accf[a][b] += __builtin_convertvector(t[b], v4f) * g;
+            } else if constexpr (WS) {
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if constexpr (!F8) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(lo4(fb8[a]), lo4(fa8[b]), acc[a][b], 0, 0, 0);
+                    const int j = (a - (TN - 2)) * TM + b;
+                    if constexpr (DMA_) {
+#pragma unroll
+                        for (int i = j * NDM8 / TAIL; i < (j + 1) * NDM8 / TAIL; ++i) dma1(ap, bp, buf, i);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    if constexpr (!F8) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(hi4(fb8[a]), hi4(fa8[b]), acc[a][b], 0, 0, 0);
+                    if constexpr (MORE_) {
+                        if (a == TN - 2 && b == 0) frag8(nbuf, TM);  // next weight fragment 0: free since block 0
+                        if (a == TN - 1) frag8(nbuf, b);              // next activation fragment b: this was its last reader
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             } else {
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
@@ -1256,6 +1294,9 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                             return launch_pipe_instance<128, 128, 2, 4, FMT, false, 4, false, false, false>(p, batch, st);
                         }
                         break;
+                    case 9:  // wave tiles of 96 x 96
+                        if (tail) break;
+                        return launch_pipe_instance<384, 192, 4, 2, FMT, false, 2, false, false, false>(p, batch, st);
                 }
             } else if constexpr (F8W) {  // fp32 accumulators are rescaled in place: every tile serves several ranges
                 switch (wcfg) {
@@ -1267,6 +1308,7 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 5: SEGQ_PIPE1(288, 192, 2, 4, true, false);
                     case 6: SEGQ_PIPE2(256, 192, 4, 2, true, false);
                     case 7: SEGQ_PIPE2(192, 256, 2, 4, true, false);
+                    case 9: SEGQ_PIPE1(384, 192, 4, 2, true, false);
                 }
             } else if (p.park) {  // int8, several ranges, a workspace to park finished ranges in: every tile
                 if constexpr (!F8W) {

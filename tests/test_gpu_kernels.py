@@ -306,7 +306,7 @@ def test_gemm_raw_accumulators(ops, tile, fa, fb, M, N, K):
         assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
 
 
-WIDE_TILES = [11, 12, 13, 14, 15, 16, 17, 18]   # the 8-wave kernels; 15 to 18 (192x288, 288x192, 256x192, 192x256) serve plain 8-bit codes only
+WIDE_TILES = [11, 12, 13, 14, 15, 16, 17, 18, 20]   # the 8-wave kernels; 15 to 18 and 20 (192x288, 288x192, 256x192, 192x256, 384x192) serve plain 8-bit codes only
 
 
 def _bf16_ulp(ref):
@@ -408,9 +408,9 @@ def test_gemm_four_stage_kernel_for_few_tokens(ops, M, N, K):
         ops.gemm(e_a, e_b, [ops.Range(0, K, None, None)], out_dtype="acc", **{**kw, "a_fmt": O.FMT_E4M3, "b_fmt": O.FMT_E4M3})
 
 
-@pytest.mark.parametrize("tile", [0, 11, 15, 16])
+@pytest.mark.parametrize("tile", [0, 11, 15, 16, 20])
 def test_gemm_more_tiles_than_compute_units(ops, tile):
-    """4608 x 4608 outputs are 324 to 384 tiles, more than the 256 CUs hold at once."""
+    """4608 x 4608 outputs are 288 to 384 tiles, more than the 256 CUs hold at once."""
     M, N, K = 4608, 4608, 256
     a = _rand_codes((M, K), O.FMT_INT8, 43)
     b = _rand_codes((N, K), O.FMT_INT8, 44)

@@ -527,10 +527,13 @@ def test_tile_and_share_choice_for_the_benchmark_shapes():
     one = lambda k: [(0, k, 0)]
     c5 = [(0, 3072, 0), (3072, 12288, 0), (3072, 12288, 1)]   # attn | MLP positive codes | MLP negative codes
     fc2 = [(0, 6144, 0), (0, 6144, 1)]
-    # configuration 3: whole rounds of 256 CUs with 192x288 / 288x192 tiles, nothing split
+    # configuration 3: whole rounds of 256 CUs with 192x288 / 384x192 / 288x192 tiles, nothing split
     assert _plan(lib, 4608, 9216, one(3072), I8)[:3] == (15, 1, 0)
-    assert _plan(lib, 4608, 12288, one(3072), I8)[:3] == (16, 1, 0)
+    assert _plan(lib, 4608, 12288, one(3072), I8)[:3] == (20, 1, 0)     # three rounds, where 288x192 needs four
+    assert _plan(lib, 4608, 12288, one(3072), F8)[:3] == (20, 1, 0)
     assert _plan(lib, 4608, 3072, one(12288), I8)[:3] == (16, 1, 0)
+    assert _plan(lib, 8192, 8192, one(8192), I8)[:3] == (11, 1, 0)      # 384 does not divide 8192
+    assert _plan(lib, 4608, 12288, [(0, 1536, 0), (1536, 1536, 0)], I8)[0] != 20   # int8 with two ranges: not on 384x192
     # configuration 1: 144 tiles of 128x128 do not fill the CUs: the four-stage kernel; fp32 output (0)
     assert _plan(lib, 256, 9216, one(1536), I8, out_dtype=0)[:3] == (19, 1, 0)
     # configuration 2: fc1 in two whole rounds of 256x192; fc2 (DualScale: two ranges) as 128 tiles in two K shares
