@@ -357,6 +357,11 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
     d.a = a.data_ptr(); d.a_neg = a_neg.data_ptr() if a_neg is not None else None; d.lda = lda
     d.b = b.data_ptr(); d.ldb = ldb
     d.out = out.data_ptr(); d.ldo = n
+    if batch == 1 and out.dim() == 2:  # a view of a wider buffer (a column slice, padded rows) is written in place
+        if out.shape != (m, n) or out.dtype != tdt or (n > 1 and out.stride(1) != 1) or (m > 1 and out.stride(0) < n):
+            raise RuntimeError("out must be an (m, n) tensor of the output dtype with contiguous rows")
+        if m > 1:
+            d.ldo = out.stride(0)
     if bias is not None:
         if bias.numel() != n or not bias.is_contiguous():
             raise RuntimeError("bias must be a contiguous vector with one entry per output column")

@@ -1174,3 +1174,51 @@ def test_empty_inputs_through_the_wrappers(ops, fmt):
     assert out.shape == (8, 0)
     torch.cuda.synchronize()
     assert bool((guard == 7.0).all())
+
+
+@pytest.mark.parametrize("pad,off", [(16, 8), (5, 3)])   # 16-byte aligned rows of the view, and not
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+def test_gemm_writes_into_a_view_of_a_wider_buffer(ops, fmt, pad, off):
+    """segq_gemm_desc.ldo larger than n: the output is a column slice of a wider row-major buffer
+    (the way fused projections are laid side by side).  Every kind of launch writes the same
+    values as into a contiguous tensor and nothing outside the slice: the general kernel, the
+    8-wave tiles incl. 384x192, K shares finished in the launch and by the second kernel, parked
+    ranges, group factors, raw accumulators and fp32 output."""
+    one = torch.ones(1, device=DEV)
+    g = torch.Generator().manual_seed(123)
+
+    def run(M, N, K, ranges_of, odt, **kw):
+        a, a2, b = _rand_codes((M, K), fmt, 50), _rand_codes((M, K), fmt, 51), _rand_codes((N, K), fmt, 52)
+        ad, a2d, bd = _to_dev_codes(a, fmt), _to_dev_codes(a2, fmt), _to_dev_codes(b, fmt)
+        sx = (torch.rand(M, generator=g) + 0.5).to(DEV)
+        sw = (torch.rand(N, generator=g) + 0.5).to(DEV)
+        rg = ranges_of(K, sx, sw)
+        bias = None if odt == "acc" else torch.randn(N, generator=g).to(DEV)
+        common = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=odt, lda=K, ldb=K, a_neg=a2d, bias=bias, **kw)
+        want = ops.gemm(ad, bd, rg, **common)
+        tdt = want.dtype
+        poison = 77 if tdt == torch.int32 else 77.0
+        buf = torch.full((M, N + pad), poison, dtype=tdt, device=DEV)
+        got = ops.gemm(ad, bd, rg, out=buf[:, off:off + N], **common)
+        torch.cuda.synchronize()
+        assert got.data_ptr() == buf[:, off:].data_ptr()
+        assert torch.equal(buf[:, off:off + N], want), (M, N, K, odt, kw)
+        assert bool((buf[:, :off] == poison).all()) and bool((buf[:, off + N:] == poison).all()), (M, N, K, odt, kw)
+
+    plain = lambda K, sx, sw: [ops.Range(0, K, sx, sw, 0, 1, 1)]
+    dual = lambda K, sx, sw: [ops.Range(0, K // 2, sx, sw, 0, 1, 1), ops.Range(K // 2, K // 2, sx, one, 0, 1, 0),
+                              ops.Range(K // 2, K // 2, sx, sw, 1, 1, 1)]
+    ws = lambda: torch.empty(64 << 20, dtype=torch.uint8, device=DEV)
+    run(70, 90, 320, plain, torch.bfloat16)                                   # general kernel
+    run(70, 90, 320, plain, "acc")
+    run(300, 700, 384, plain, torch.bfloat16, tile=11)
+    run(300, 700, 384, plain, torch.float32, tile=15)
+    run(400, 200, 256, plain, torch.bfloat16, tile=20)
+    run(400, 200, 256, plain, "acc", tile=20)
+    run(300, 200, 2048, plain, torch.bfloat16, tile=17, split_k=2, workspace=ws())   # finished in the launch
+    run(300, 200, 2048, plain, torch.float16, tile=17, split_k=4, workspace=ws())    # summed by the second kernel
+    run(300, 200, 1024, dual, torch.bfloat16, tile=16 if fmt == O.FMT_E4M3 else 11, workspace=ws())  # rescaled in place / parked
+    run(300, 200, 1024, dual, torch.bfloat16)                                  # the library's choice without a workspace
+    if fmt == O.FMT_INT8:
+        fac = (torch.rand(1024 // 128, 200, generator=g) + 0.5).to(DEV)
+        run(300, 200, 1024, lambda K, sx, sw: [ops.Range(0, K, sx, one, 0, 1, 0)], torch.bfloat16, group_dequant=fac)
