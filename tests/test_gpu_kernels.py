@@ -1222,3 +1222,55 @@ def test_gemm_writes_into_a_view_of_a_wider_buffer(ops, fmt, pad, off):
     if fmt == O.FMT_INT8:
         fac = (torch.rand(1024 // 128, 200, generator=g) + 0.5).to(DEV)
         run(300, 200, 1024, lambda K, sx, sw: [ops.Range(0, K, sx, one, 0, 1, 0)], torch.bfloat16, group_dequant=fac)
+
+
+@pytest.mark.parametrize("fa,fb", [(O.FMT_INT8, O.FMT_INT8), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_INT8, O.FMT_INT4)])
+def test_gemm_reads_operands_from_views_of_wider_buffers(ops, fa, fb):
+    """lda and ldb larger than K: both code matrices (and the second activation tensor) are column
+    slices, at 16-byte offsets, of wider row-major buffers whose other columns hold other codes.
+    Same result as from contiguous copies on the general kernel, the 8-wave tiles, K shares, parked /
+    rescaled ranges and group factors."""
+    one = torch.ones(1, device=DEV)
+    g = torch.Generator().manual_seed(321)
+    w4 = fb == O.FMT_INT4
+
+    def run(M, N, K, ranges_of, odt, **kw):
+        a, a2, b = _rand_codes((M, K), fa, 60), _rand_codes((M, K), fa, 61), _rand_codes((N, K), fb, 62)
+        ad, a2d, bd = _to_dev_codes(a, fa), _to_dev_codes(a2, fa), _to_dev_codes(b, fb)   # bd: (N, K / 2) bytes when int4
+        if bd.dim() == 1:
+            bd = bd.view(N, -1)
+        def widen(t, left, right, seed):
+            wide = torch.from_numpy(np.random.default_rng(seed).integers(0, 120, size=(t.shape[0], left + t.shape[1] + right))
+                                    .astype(np.uint8)).to(DEV).view(t.dtype)
+            wide[:, left:left + t.shape[1]] = t
+            return wide, wide[:, left:left + t.shape[1]]
+        abuf, av = widen(ad, 32, 48, 1)
+        a2buf, a2v = widen(a2d, 32, 48, 2)       # same stride as a: one lda serves both
+        bbuf, bv = widen(bd, 16, 16, 3)
+        sx = (torch.rand(M, generator=g) + 0.5).to(DEV)
+        sw = (torch.rand(N, generator=g) + 0.5).to(DEV)
+        rg = ranges_of(K, sx, sw)
+        bias = None if odt == "acc" else torch.randn(N, generator=g).to(DEV)
+        common = dict(m=M, n=N, a_fmt=fa, b_fmt=fb, out_dtype=odt, bias=bias, **kw)
+        want = ops.gemm(ad, bd, rg, lda=K, ldb=bd.shape[1], a_neg=a2d, **common)
+        got = ops.gemm(av, bv, rg, lda=abuf.stride(0), ldb=bbuf.stride(0), a_neg=a2v, **common)
+        assert av.data_ptr() % 16 == 0 and bv.data_ptr() % 16 == 0
+        assert torch.equal(got, want), (M, N, K, odt, kw)
+
+    plain = lambda K, sx, sw: [ops.Range(0, K, sx, sw, 0, 1, 1)]
+    dual = lambda K, sx, sw: [ops.Range(0, K // 2, sx, sw, 0, 1, 1), ops.Range(K // 2, K // 2, sx, one, 0, 1, 0),
+                              ops.Range(K // 2, K // 2, sx, sw, 1, 1, 1)]
+    ws = lambda: torch.empty(64 << 20, dtype=torch.uint8, device=DEV)
+    run(70, 90, 320, plain, torch.bfloat16)
+    run(70, 90, 320, plain, "acc")
+    run(300, 700, 384, plain, torch.bfloat16, tile=11)
+    run(300, 200, 1024, dual, torch.bfloat16)
+    run(300, 200, 1024, dual, torch.bfloat16, workspace=ws())
+    if not w4:
+        run(400, 200, 256, plain, torch.bfloat16, tile=20)
+        run(300, 700, 384, plain, torch.float32, tile=15)
+        run(300, 200, 2048, plain, torch.bfloat16, tile=17, split_k=2, workspace=ws())
+        run(300, 200, 2048, plain, torch.float16, tile=17, split_k=4, workspace=ws())
+    if fa == O.FMT_INT8:
+        fac = (torch.rand(1024 // 128, 200, generator=g) + 0.5).to(DEV)
+        run(300, 200, 1024, lambda K, sx, sw: [ops.Range(0, K, sx, one, 0, 1, 0)], torch.bfloat16, group_dequant=fac, workspace=ws())
