@@ -1274,3 +1274,40 @@ def test_gemm_reads_operands_from_views_of_wider_buffers(ops, fa, fb):
     if fa == O.FMT_INT8:
         fac = (torch.rand(1024 // 128, 200, generator=g) + 0.5).to(DEV)
         run(300, 200, 1024, lambda K, sx, sw: [ops.Range(0, K, sx, one, 0, 1, 0)], torch.bfloat16, group_dequant=fac, workspace=ws())
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_quantize_reads_and_writes_views_of_wider_buffers(ops, fmt, dt):
+    """ldx, ld_codes and ld_gate larger than cols: the input (a GEGLU projection's value half, the
+    gate being the other half of the same buffer) and the codes (one K segment of a wider code
+    matrix) are column slices.  Same codes and scales as from contiguous copies for static,
+    dynamic and DualScale launches on each dynamic kernel, and nothing written outside the slice."""
+    g = torch.Generator().manual_seed(55)
+    for K in (256, 3072, 4800, 12288):      # flat / one wave per row and workgroup / one wave per row / one workgroup per row
+        M = 9
+        wide = (torch.randn(M, 2 * K + 32, generator=g) * 2).to(TDT[dt]).to(DEV)
+        x, gate = wide[:, 16:16 + K], wide[:, 16 + K:16 + 2 * K]     # 32- or 64-byte offsets
+        xc, gc = x.contiguous(), gate.contiguous()
+        ccols = K // 2 if fmt == O.FMT_INT4 else K
+        for kind in ("static", "dynamic", "dual", "gated"):
+            poison = 0x55
+            cbuf = torch.full((M, ccols + 48), poison, dtype=torch.uint8, device=DEV).view(ops.code_dtype(fmt))
+            cview = cbuf[:, 16:16 + ccols]
+            mk = lambda: torch.empty(M, device=DEV)
+            if kind == "static":
+                s = torch.full((1,), 11.0, device=DEV)
+                want = ops.quantize(xc, fmt, s)
+                got = ops.quantize(x, fmt, s, out=cview)
+            else:
+                kw = dict(row_stride=1, dynamic=True, dual=kind == "dual")
+                if kind == "gated":
+                    kw.update(pre_op="gelu_tanh")
+                s1, n1, s2, n2 = mk(), (mk() if kind == "dual" else None), mk(), (mk() if kind == "dual" else None)
+                want = ops.quantize(xc, fmt, s1, n1, gate=gc if kind == "gated" else None, **kw)
+                got = ops.quantize(x, fmt, s2, n2, gate=gate if kind == "gated" else None, out=cview, **kw)
+                assert torch.equal(s1, s2) and (n1 is None or torch.equal(n1, n2)), (K, kind)
+            torch.cuda.synchronize()
+            assert torch.equal(cview, want), (K, kind)
+            raw = cbuf.view(torch.uint8)
+            assert bool((raw[:, :16] == poison).all()) and bool((raw[:, 16 + ccols:] == poison).all()), (K, kind)
