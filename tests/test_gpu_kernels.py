@@ -1311,3 +1311,37 @@ def test_quantize_reads_and_writes_views_of_wider_buffers(ops, fmt, dt):
             assert torch.equal(cview, want), (K, kind)
             raw = cbuf.view(torch.uint8)
             assert bool((raw[:, :16] == poison).all()) and bool((raw[:, 16 + ccols:] == poison).all()), (K, kind)
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+def test_gemm_split_k_on_the_384x192_tile(ops, fmt):
+    """Tile 20 by id with its K steps shared by 2, 3 and 5 workgroups (the second kernel sums the
+    shares): one range in both formats, and in e4m3 three ranges rescaled in place, against the
+    unsplit launch and the closed form; int8 with several ranges is refused there."""
+    M, N, K0, K1 = 400, 210, 384, 640
+    K = K0 + K1
+    a, a2, b = _rand_codes((M, K), fmt, 71), _rand_codes((M, K), fmt, 72), _rand_codes((N, K), fmt, 73)
+    ad, a2d, bd = (_to_dev_codes(t, fmt) for t in (a, a2, b))
+    g = torch.Generator().manual_seed(74)
+    sx, sx2 = torch.rand(M, generator=g) + 0.5, torch.rand(M, generator=g) + 0.5
+    sw, bias = torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+    one = [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
+    three = [ops.Range(0, K0, sx2.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(K0, K1, sx.to(DEV), sw.to(DEV), 0, 1, 1),
+             ops.Range(K0, K1, sx2.to(DEV), sw.to(DEV), 1, 1, 1)]
+    ws = torch.empty(ops.split_bytes(M, N, 8, park=True), dtype=torch.uint8, device=DEV)
+    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, bias=bias.to(DEV), a_neg=a2d, tile=20, workspace=ws)
+    av, a2v, bv = (O.code_values(t, fmt) for t in (a, a2, b))
+    f64 = lambda t: t.numpy().astype(np.float64)
+    want1 = av @ bv.T / (f64(sx)[:, None] * f64(sw)[None, :]) + f64(bias)
+    want3 = (av[:, :K0] @ bv[:, :K0].T / (f64(sx2)[:, None] * f64(sw)[None, :]) + av[:, K0:] @ bv[:, K0:].T / (f64(sx)[:, None] * f64(sw)[None, :]) +
+             a2v[:, K0:] @ bv[:, K0:].T / (f64(sx2)[:, None] * f64(sw)[None, :]) + f64(bias))
+    tol = 5e-6 if fmt == O.FMT_INT8 else 1e-3
+    for rg, want in ((one, want1), (three, want3)):
+        if rg is three and fmt == O.FMT_INT8:
+            with pytest.raises(RuntimeError):
+                ops.gemm(ad, bd, rg, out_dtype=torch.float32, split_k=1, **kw)
+            continue
+        for sk in (1, 2, 3, 5):
+            out = ops.gemm(ad, bd, rg, out_dtype=torch.float32, split_k=sk, **kw)
+            assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max(), (len(rg), sk)
+            assert ops.gemm_plan(ops.gemm_desc(ad, bd, rg, out_dtype=torch.float32, split_k=sk, **kw), ws)["splits"] == sk
