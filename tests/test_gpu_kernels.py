@@ -1345,3 +1345,30 @@ def test_gemm_split_k_on_the_384x192_tile(ops, fmt):
             out = ops.gemm(ad, bd, rg, out_dtype=torch.float32, split_k=sk, **kw)
             assert np.abs(_np(out).astype(np.float64) - want).max() <= tol * np.abs(want).max(), (len(rg), sk)
             assert ops.gemm_plan(ops.gemm_desc(ad, bd, rg, out_dtype=torch.float32, split_k=sk, **kw), ws)["splits"] == sk
+
+
+@pytest.mark.parametrize("fa,fb", [(O.FMT_INT8, O.FMT_INT8), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_INT8, O.FMT_INT4)])
+def test_gemm_smallest_problems(ops, fa, fb):
+    """One row, one column, the shortest contraction (16, or 32 with int4 weights), on the library's
+    own choice and on the smallest general and 8-wave tiles: raw sums and the fused output."""
+    kmin = 32 if fb == O.FMT_INT4 else 16
+    g = torch.Generator().manual_seed(9)
+    for M, N, K in ((1, 1, kmin), (1, 16, kmin), (17, 1, 2 * kmin), (1, 130, 128), (2, 3, 256)):
+        a, b = _rand_codes((M, K), fa, 90), _rand_codes((N, K), fb, 91)
+        ad, bd = _to_dev_codes(a, fa), _to_dev_codes(b, fb)
+        ldb = K // 2 if fb == O.FMT_INT4 else K
+        ref = O.gemm_acc(a, b, fa, fb).astype(np.float64)
+        sx, sw, bias = torch.rand(M, generator=g) + 0.5, torch.rand(N, generator=g) + 0.5, torch.randn(N, generator=g)
+        want = ref / (sx.numpy().astype(np.float64)[:, None] * sw.numpy().astype(np.float64)[None, :]) + bias.numpy()
+        mag = np.abs(O.code_values(a, fa)) @ np.abs(O.code_values(b, fb)).T if fa == O.FMT_E4M3 else 0.0
+        for tile in (0, 4, 14):
+            if tile == 14 and K % 128:   # the 8-wave tiles take K in whole 128-byte steps
+                continue
+            kw = dict(m=M, n=N, a_fmt=fa, b_fmt=fb, lda=K, ldb=ldb, tile=tile)
+            out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
+            assert out.shape == (M, N)
+            assert (np.abs(out.cpu().numpy().astype(np.float64) - ref) <= FP8_ACC_TOL * mag + 1e-30).all(), (M, N, K, tile)
+            for odt, tol in ((torch.float32, 2e-6), (torch.bfloat16, 2.0 ** -8)):
+                y = ops.gemm(ad, bd, [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)], out_dtype=odt, bias=bias.to(DEV), **kw)
+                slack = FP8_ACC_TOL * mag / (sx.numpy()[:, None] * sw.numpy()[None, :]) if fa == O.FMT_E4M3 else 0.0
+                assert (np.abs(_np(y).astype(np.float64) - want) <= tol * np.abs(want) + slack + 1e-30).all(), (M, N, K, tile, odt)
