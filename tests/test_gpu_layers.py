@@ -407,3 +407,26 @@ def test_zero_tokens_give_an_empty_output(config):
         assert chunks.shape[-2] == 0
     torch.cuda.synchronize()
     assert torch.equal(layer(xin), want)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_leading_batch_dimensions(config):
+    """(batch, tokens, features) and (a, b, tokens, features) inputs, as the transformer blocks pass
+    them: the same values as the flattened 2-D call, in the input's leading shape, on both routes;
+    a non-contiguous view (every second token) too."""
+    from segquant_amd import workloads as W
+    for spec in W.config_linears(config, M=96)[:2]:
+        layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+        x2 = x.to(spec.x_dtype).to(DEV)
+        want = layer(x2)
+        for shape in ((2, 48), (2, 3, 16), (1, 96), (96, 1)):
+            out = layer(x2.reshape(*shape, spec.K))
+            assert out.shape == (*shape, spec.N) and out.dtype == spec.x_dtype
+            assert torch.equal(out.reshape(96, spec.N), want), (spec.name, shape)
+        every_second = torch.stack([x2, -x2], dim=1)[:, 0]      # rows 2 K apart in memory
+        assert not every_second.is_contiguous()
+        assert torch.equal(layer(every_second), want), spec.name
+        if config in (1, 2, 3):
+            chunks2 = layer(x2, chunked=True)
+            chunks3 = layer(x2.reshape(2, 48, spec.K), chunked=True)
+            assert torch.equal(chunks3.reshape(chunks2.shape), chunks2), spec.name
