@@ -430,3 +430,22 @@ def test_leading_batch_dimensions(config):
             chunks2 = layer(x2, chunked=True)
             chunks3 = layer(x2.reshape(2, 48, spec.K), chunked=True)
             assert torch.equal(chunks3.reshape(chunks2.shape), chunks2), spec.name
+
+
+@pytest.mark.parametrize("config", [2, 3, 5])
+def test_one_layer_serves_every_float_input_dtype(config):
+    """The reference's models run in fp16; the benchmark configurations in bf16 and fp32.  One
+    calibrated layer takes all three: the output comes back in the input's dtype and differs from
+    the fp32 call by that dtype's rounding of input and output only (the codes of an fp16 or bf16
+    input are those of the rounded values, so the comparison is against the fp32 call on the
+    rounded input)."""
+    from segquant_amd import workloads as W
+    spec = W.config_linears(config, M=80)[0]
+    layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+    for dt, ulp in ((torch.float16, 2.0 ** -11), (torch.bfloat16, 2.0 ** -8), (torch.float32, 0.0)):
+        xin = x.to(dt).to(DEV)
+        out = layer(xin)
+        assert out.dtype == dt and out.shape == (80, spec.N)
+        ref = layer(xin.float())           # the same rounded values, fp32 in and out
+        err = (out.float() - ref).abs().max().item() / ref.abs().max().item()
+        assert err <= ulp + 1e-6, (spec.name, dt, err)
