@@ -84,7 +84,10 @@ const char* segq_last_error(void);
  * dynamic != 0: scale[] (and scale_neg[]) are OUTPUTS.  The kernel takes the
  * absolute maximum of every (row, column segment), writes
  * qmax / max(amax, 2^-24) there (segquant/quantizers/quantizer.py:211-219;
- * dual: :183-203; e4m3: 448) and quantises with it.  Needs row_stride == 1 or a
+ * dual: :183-203; e4m3: 448) and quantises with it.  A NaN in the segment makes a
+ * single scale NaN, as torch's amax does (and every code of the segment the NaN
+ * code); the two DualScale maxima are taken over x > 0 and x < 0, where a NaN is on
+ * neither side; an infinite maximum gives scale 0.  Needs row_stride == 1 or a
  * single row per scale; has no counterpart kernel in the reference, whose
  * dynamic mode calls a method that does not exist (optimum/optimizer.py:96-100).
  *
