@@ -102,6 +102,12 @@ def main():
     ap.add_argument("--overlap", action="store_true",
                     help="also time the steps with each linear's quantise kernel on a second stream under the previous linear's "
                          "GEMM (measured on config 3: 7 %% slower than in sequence, the chip being held by its power limit)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the steps replayed from captured HIP graphs (one graph per rotating input set, at most 32): "
+                         "what a serving loop pays when the host's enqueue time is off the path")
+    ap.add_argument("--pair", action="store_true",
+                    help="config 2 only: also time fc1 -> GELU(tanh) -> fc2 as chained linears (forward_into: fc1's GEMM epilogue writes "
+                         "fc2's DualScale codes; no float tensor and no quantise launch between the two GEMMs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")
     args = ap.parse_args()
@@ -201,6 +207,56 @@ def main():
             step_overlapped(args.warmup + i)
         torch.cuda.synchronize()
         wall_ov = time.perf_counter() - t2
+    graph_res = None
+    if args.graph:
+        n_g = min(n_sets, 32)
+        cap = torch.cuda.Stream()
+        cap.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(cap):  # buffers, workspaces and kernel attributes of this stream exist before the capture
+            for i in range(2):
+                step(i)
+        torch.cuda.current_stream().wait_stream(cap)
+        torch.cuda.synchronize()
+        graphs = []
+        for i in range(n_g):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=cap):
+                step(i)
+            graphs.append(gr)
+        for i in range(args.warmup):
+            graphs[i % n_g].replay()
+        torch.cuda.synchronize()
+        tg0 = time.perf_counter()
+        for i in range(args.steps):
+            graphs[i % n_g].replay()
+        torch.cuda.synchronize()
+        wall_g = time.perf_counter() - tg0
+        graph_res = {"value": round(total_ops * args.steps / wall_g / 1e12, 2), "unit": "TOP/s", "ms_per_step": round(wall_g / args.steps * 1e3, 4),
+                     "graphs": n_g, "how": "each step replayed from a HIP graph captured over one of the rotating input sets"}
+        del graphs
+    pair_res = None
+    if args.pair and args.config == 2:
+        fc1, fc2 = layers
+        xs1 = [s_[0] for s_ in sets]
+        for i in range(args.warmup):
+            fc1.forward_into(fc2, xs1[i % n_sets], pre_op="gelu_tanh")
+        torch.cuda.synchronize()
+        tp0 = time.perf_counter()
+        for i in range(args.steps):
+            fc1.forward_into(fc2, xs1[i % n_sets], pre_op="gelu_tanh")
+        torch.cuda.synchronize()
+        wall_p = time.perf_counter() - tp0
+        with ops.record_launches() as plog:
+            for i in range(args.steps):
+                fc1.forward_into(fc2, xs1[i % n_sets], pre_op="gelu_tanh")
+            torch.cuda.synchronize()
+        per = {}
+        for j, (kind, e0, e1, info) in enumerate(plog):
+            per.setdefault(("fc1_quantize", "fc1_gemm_codes_out", "fc2_gemm")[j % 3], []).append(e0.elapsed_time(e1) * 1e3)
+        pair_res = {"value": round(total_ops * args.steps / wall_p / 1e12, 2), "unit": "TOP/s", "ms_per_step": round(wall_p / args.steps * 1e3, 4),
+                    "launches_per_step": 3, "quantize_launches_per_step": 1,
+                    "kernel_us": {k: round(sum(v) / len(v), 2) for k, v in per.items()},
+                    "how": "fc1.forward_into(fc2, x, pre_op='gelu_tanh'): fc1 quantise, fc1 GEMM writing fc2's two code tensors, fc2 GEMM"}
     # Per-kernel durations for the roofline figures, outside the timed region.  GEMM: the same
     # steps with a HIP event pair around every launch (the records cost a few microseconds per
     # launch, little against a GEMM).  Quantise: the kernels are ~10-30 us, so each linear's
@@ -293,6 +349,14 @@ def main():
         kernels.append(plan["kernel"] + (f" x{plan['splits']} K shares" if plan["splits"] > 1 else "") + (" parked ranges" if plan["parked"] else ""))
     fmt = specs[0].act
     peak = PEAK_TOPS[fmt]
+    # the same peak from the device itself: CUs x 4 SIMDs x 2048 8-bit ops per clock and SIMD (one
+    # 16x16x64 int8 or 16x16x128 fp8 MFMA every 16 / 32 clocks) x the highest engine clock it reports
+    import ctypes
+    from segquant_amd import _lib as L_
+    dev_cus, dev_khz = ctypes.c_int32(0), ctypes.c_int32(0)
+    L_.check(lib().segq_device_info(ctypes.byref(dev_cus), ctypes.byref(dev_khz)))
+    clock_ghz = dev_khz.value / 1e6
+    peak_dev = dev_cus.value * 4 * 2048 * clock_ghz / 1e3
     g_tops = g_ops / g_t / 1e12
     q_gbs = q_bytes / q_t / 1e9
     traffic, traffic_source = recorded_traffic(args.config)
@@ -307,6 +371,8 @@ def main():
                    "input_dtype": str(specs[0].x_dtype).replace("torch.", ""), "output_dtype": str(specs[0].x_dtype).replace("torch.", "")},
         "roofline": {"bound": "mfma", "kernel": " / ".join(dict.fromkeys(kernels)) + f" ({fmt})", "achieved": round(g_tops, 2), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(g_tops / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "peak_from_device": {"compute_units": dev_cus.value, "max_engine_clock_GHz": round(clock_ghz, 3),
+                                          "ops_per_clock_per_cu": 8192, "TOP/s": round(peak_dev, 1)},
                      "launches": n_g, "avg_launch_us": round(g_t / max(n_g, 1) * 1e6, 2),
                      "algorithmic_bytes_per_launch": round(g_bytes / max(n_g, 1)),
                      "executed_tops": round(g_exec / g_t / 1e12, 2),
@@ -349,6 +415,11 @@ def main():
             res.append({"linear": sp.name, **{k: round(v, 1) for k, v in t.items()}})
             del parts
         out["producer_fusion_us"] = res
+    if graph_res is not None:
+        out["graph_replay"] = graph_res
+    if pair_res is not None:
+        out["chained_pair"] = pair_res
+    out["quantize"]["launches_per_step"] = len(layers)
     if wall_ov is not None:
         out["overlapped"] = {"value": round(total_ops * args.steps / wall_ov / 1e12, 2), "unit": "TOP/s",
                              "ms_per_step": round(wall_ov / args.steps * 1e3, 4),

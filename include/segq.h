@@ -291,6 +291,28 @@ typedef struct segq_gemm_desc {
     const void* lowrank_l2t; /* device: (n, lowrank_rank), i.e. L2 transposed, the contraction index contiguous */
     int64_t ld_lowrank_l2t;
     int32_t lowrank_rank;   /* multiple of 32, at most 512; 0 with lowrank_t == NULL */
+    int32_t out_pre_op;     /* segq_pre_op applied to the result before it is encoded (out_codes only) */
+    void* out_codes;        /* device or NULL.  When set, the launch writes CODES instead of floats: the (m, n)
+                         * code tensor that segq_quantize would make of this GEMM's output for the linear that
+                         * follows, so that neither the float output is written nor a quantise launch reads it
+                         * back.  Every result is rounded to out_dtype (the dtype the output tensor would have
+                         * had), out_pre_op is applied and rounded to out_dtype again, the value is multiplied by
+                         * out_scale[0] and encoded as out_code_fmt: bit for bit the codes of segq_gemm followed
+                         * by segq_quantize with pre_op and a static per-tensor scale.  With out_scale_neg set
+                         * (DualScale) out_codes_neg is required: values >= 0 go to out_codes scaled by
+                         * out_scale[0], the others to out_codes_neg scaled by out_scale_neg[0], the tensor not
+                         * taken holding code(0) (segquant/src/real_quant/quantizer.cuh:178-206).  out is
+                         * ignored (may be NULL).  Needs plain int8 or e4m3 codes on both sides, one range with K
+                         * a multiple of 128, batch == 1, out_dtype F16 or BF16; no split_k, group factors or
+                         * low-rank branch (SEGQ_ERR_UNSUPPORTED otherwise).
+                         * These are the reference's chained linears, which there pass a full-size tensor
+                         * through an activation kernel and a quantise kernel between the two GEMMs
+                         * (backend/torch/layers/activations.py:52-57 feeding real_gemm.cu:700-705). */
+    void* out_codes_neg;
+    int64_t ld_out_codes;   /* bytes; >= n */
+    const float* out_scale; /* device: one float */
+    const float* out_scale_neg; /* device or NULL */
+    int32_t out_code_fmt;   /* SEGQ_CODE_I8 | SEGQ_CODE_E4M3 */
     int32_t reserved2;
     segq_krange ranges[SEGQ_MAX_RANGES];
 } segq_gemm_desc;
@@ -324,8 +346,12 @@ int segq_gemm_plan(const segq_gemm_desc* d, int32_t* tile, int32_t* splits, int3
  * segq_gemm called with a workspace of segq_gemm_workspace_bytes(d) bytes, but the workspace
  * (expanded int4 weights, parked sums of int8 ranges, split-K partial results) is an array of
  * SEGQ_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, from the
- * first use on that GPU until the process ends; d->workspace is ignored.  A launch that would
- * use more than that is refused with SEGQ_ERR_ARG and a message (nothing is enqueued).  The call
+ * first use on that GPU until the process ends; d->workspace is ignored.  A launch that could
+ * use more than that runs with what fits, exactly as segq_gemm does when it is lent a workspace
+ * of SEGQ_NOALLOC_SCRATCH_BYTES (fewer K shares; int8 ranges summed in a second register set
+ * on smaller tiles instead of parked: the same result up to the order of fp32 additions); only
+ * a launch that cannot run with less (an explicit split_k, group factors with int4 weights
+ * beyond the array) is refused, with its status and a message, and nothing is enqueued.  The call
  * allocates nothing and frees nothing; the array's address on the current device is resolved on
  * the first call there, or ahead of time by segq_init().
  *
@@ -341,6 +367,12 @@ int64_t segq_noalloc_scratch_bytes(void); /* SEGQ_NOALLOC_SCRATCH_BYTES of the l
  * properties and resolves the scratch array's address there, which the entry points otherwise do
  * on their first call on that device.  No counterpart in the reference. */
 int segq_init(void);
+
+/* Compute units and highest engine clock (kHz) of the current device, as the HIP runtime reports
+ * them: what the dense 8-bit MFMA peak follows from (compute units x 4 SIMDs x 2048 operations per
+ * clock x clock).  For benchmarks that state the peak they measure against; no counterpart in the
+ * reference.  Either pointer may be NULL. */
+int segq_device_info(int32_t* compute_units, int32_t* max_engine_clock_khz);
 
 /* Quantise-then-multiply in one call: q writes its codes into a caller-provided
  * workspace that g reads as its a (and a_neg).  Replaces the body of

@@ -58,7 +58,9 @@ class GemmDesc(C.Structure):
         ("group_dequant", C.c_void_p), ("group_dequant_stride", C.c_int64),
         ("addend", C.c_void_p), ("ld_addend", C.c_int64), ("split_k", C.c_int64),
         ("lowrank_t", C.c_void_p), ("ld_lowrank_t", C.c_int64), ("lowrank_l2t", C.c_void_p), ("ld_lowrank_l2t", C.c_int64),
-        ("lowrank_rank", C.c_int32), ("reserved2", C.c_int32),
+        ("lowrank_rank", C.c_int32), ("out_pre_op", C.c_int32),
+        ("out_codes", C.c_void_p), ("out_codes_neg", C.c_void_p), ("ld_out_codes", C.c_int64),
+        ("out_scale", C.c_void_p), ("out_scale_neg", C.c_void_p), ("out_code_fmt", C.c_int32), ("reserved2", C.c_int32),
         ("ranges", KRange * SEGQ_MAX_RANGES),
     ]
 
@@ -66,7 +68,7 @@ class GemmDesc(C.Structure):
 EXPORTS = (
     "segq_version", "segq_last_error", "segq_quantize", "segq_quantize_many", "segq_quantize_weights_scalar",
     "segq_quantize_weights_rows", "segq_quantize_weights_groups", "segq_repack_int4_cols_to_rows", "segq_gemm", "segq_gemm_tile_count", "segq_gemm_workspace_bytes", "segq_gemm_plan", "segq_linear", "segq_fake_e4m3",
-    "segq_gemm_noalloc", "segq_noalloc_scratch_bytes", "segq_init",
+    "segq_gemm_noalloc", "segq_noalloc_scratch_bytes", "segq_init", "segq_device_info",
 )
 
 _lib = None
@@ -117,6 +119,8 @@ def lib() -> C.CDLL:
     L.segq_gemm_noalloc.restype = C.c_int
     L.segq_noalloc_scratch_bytes.restype = C.c_int64
     L.segq_init.restype = C.c_int
+    L.segq_device_info.argtypes = [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    L.segq_device_info.restype = C.c_int
     L.segq_linear.argtypes = [C.POINTER(QuantDesc), C.POINTER(GemmDesc), C.c_void_p]
     L.segq_fake_e4m3.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_void_p]
     for name in ("segq_quantize", "segq_quantize_weights_scalar", "segq_quantize_weights_rows", "segq_gemm",

@@ -200,7 +200,15 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     if (d->m < 0 || d->n < 0 || d->batch < 1) return fail(SEGQ_ERR_ARG, "segq_gemm: bad sizes");
     if (d->m == 0 || d->n == 0) return SEGQ_OK;
     if (d->m > 0x7fffffff / 2 || d->n > 0x7fffffff / 2) return fail(SEGQ_ERR_ARG, "segq_gemm: m or n too large");
-    if (!d->a || !d->b || !d->out) return fail(SEGQ_ERR_ARG, "segq_gemm: null a, b or out");
+    const bool codes_out = d->out_codes != nullptr;
+    if (!d->a || !d->b || (!d->out && !codes_out)) return fail(SEGQ_ERR_ARG, "segq_gemm: null a, b or out");
+    if (codes_out) {
+        if ((d->out_dtype != SEGQ_BF16 && d->out_dtype != SEGQ_F16) || d->batch != 1 || !d->out_scale || d->ld_out_codes < d->n || d->split_k > 1 ||
+            (d->out_code_fmt != SEGQ_CODE_I8 && d->out_code_fmt != SEGQ_CODE_E4M3) || d->out_pre_op < 0 || d->out_pre_op > SEGQ_PRE_SILU ||
+            (d->out_scale_neg != nullptr) != (d->out_codes_neg != nullptr))
+            return fail(SEGQ_ERR_ARG, "segq_gemm: out_codes needs out_dtype F16 or BF16, batch == 1, ld_out_codes >= n, int8 or e4m3 codes, "
+                                      "out_scale, and out_scale_neg together with out_codes_neg");
+    }
     if (d->n_ranges < 1 || d->n_ranges > SEGQ_MAX_RANGES) return fail(SEGQ_ERR_ARG, "segq_gemm: n_ranges %d out of range", d->n_ranges);
     const bool i8 = d->a_fmt == SEGQ_CODE_I8 && d->b_fmt == SEGQ_CODE_I8;
     const bool f8 = d->a_fmt == SEGQ_CODE_E4M3 && d->b_fmt == SEGQ_CODE_E4M3;
@@ -212,7 +220,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     if (d->lda % 16 || d->ldb % 16 || !al(d->a, 16) || !al(d->b, 16) || (d->a_neg && !al(d->a_neg, 16)) ||
         d->batch_stride_a % 16 || d->batch_stride_b % 16)
         return fail(SEGQ_ERR_ARG, "segq_gemm: a and b need 16-byte aligned bases and row strides");
-    if (d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
+    if (!codes_out && d->ldo < d->n) return fail(SEGQ_ERR_ARG, "segq_gemm: ldo smaller than n");
     if (d->addend && (d->out_dtype == SEGQ_ACC || d->ld_addend < d->n))
         return fail(SEGQ_ERR_ARG, "segq_gemm: an addend needs a float output and ld_addend >= n");
     const bool lowrank = d->lowrank_t != nullptr || d->lowrank_rank != 0;
@@ -397,7 +405,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     int64_t part_bytes = 0;
     {
         const bool can = plain8 && wide_ok && d->batch == 1 && !groups && !lowrank && d->out_dtype != SEGQ_ACC && ws && al(ws, 16) &&
-                         d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG);
+                         d->split_k != 1 && (d->tile == 0 || cfg >= FIRST_WIDE_CFG) && !codes_out;
         const int64_t total_steps = ktotal / 128;
         if (d->split_k > 1 && !can)
             return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: split_k needs plain 8-bit codes, K ranges in multiples of 128, one problem, "
@@ -488,6 +496,24 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         p.lr_ldl = d->ld_lowrank_l2t;
         p.lr_rank = d->lowrank_rank;
     }
+    if (codes_out) {
+        // the epilogue that writes codes is built into two tiles of the pipelined kernels
+        if (!(plain8 && wide_ok && !fold && !groups && !lowrank && splits == 1))
+            return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: out_codes needs plain int8 or e4m3 codes on both sides and one K range in "
+                                              "multiples of 128; no group factors, low-rank branch or split_k");
+        // 128 x 128: two workgroups share a CU, so one's epilogue (all VALU: ~40 instructions per element
+        // with a GELU and two code tensors) can run under the other's MFMAs.  Measured on 4096 x 1536 ->
+        // 6144 e4m3, GELU(tanh), DualScale: 66 us against 104 us on 256 x 256, one workgroup per CU
+        if (d->tile == 0) cfg = FIRST_WIDE_CFG + 3;
+        p.oc = d->out_codes;
+        p.oc_neg = d->out_codes_neg;
+        p.ldoc = d->ld_out_codes;
+        p.oc_scale = d->out_scale;
+        p.oc_scale_neg = d->out_scale_neg;
+        p.oc_fmt = d->out_code_fmt;
+        p.oc_pre = d->out_pre_op;
+        p.oc_vec = d->ld_out_codes % 8 == 0 && al(d->out_codes, 8) && (!d->out_codes_neg || al(d->out_codes_neg, 8));
+    }
     const TileCfg& c = TILE_CFGS[cfg];
     p.tiles_m = (int32_t)((d->m + c.bm - 1) / c.bm);
     p.tiles_n = (int32_t)((d->n + c.bn - 1) / c.bn);
@@ -496,12 +522,20 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         plan->tile = cfg + 1;
         plan->splits = splits;
         plan->parked = park ? 1 : 0;
-        return SEGQ_OK;
+        // walk the same dispatch the launch takes, down to the kernel instance, and launch nothing:
+        // the plan is refused exactly when the launch would be
+        p.dry = 1;
     }
     // tiles are numbered down groups of this many tile rows, so that the 32 tiles an XCD holds at a time
     // share few operand panels; 384-row tiles reach that with half as many rows (e4m3 4608 x 12288 x 3072
     // 140.7 -> 136.2 us; other heights between 2 and 16 measured the same or worse on the 4608-token shapes)
     p.group_m = (cfg == FIRST_WIDE_CFG + 9) ? 4 : 8;
+    {
+        // e4m3 only (4608 x 15360 x 3072 in three ranges: 350 -> 338 us); int8, which parks its sums at the
+        // boundaries, loses more to the XCDs reading different operand columns at a time than it gains
+        // from spreading its stores (385 -> 397 us), and keeps the common order
+        p.rot = (d->n_ranges > 1 && splits == 1 && f8) ? 1 : 0;
+    }
     if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff || d->batch > 65535) return fail(SEGQ_ERR_ARG, "segq_gemm: grid too large");
     const int64_t osz = (d->out_dtype == SEGQ_F32 || d->out_dtype == SEGQ_ACC) ? 4 : 2;
     p.vec_store = ((d->ldo * osz) % (4 * osz) == 0) && ((d->batch_stride_out * osz) % (4 * osz) == 0) && al(d->out, 4 * osz);
@@ -513,7 +547,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         p.arrived = reinterpret_cast<unsigned int*>(static_cast<uint8_t*>(d->workspace) + tiles * 2 * c.bm * c.bn * 4);
         p.bsA = p.bsB = p.bsC = p.bsSx = p.bsSw = 0;  // blockIdx.y counts shares here, not problems
         static unsigned int g_stamp = 0x5e690000u;
-        do p.stamp = __atomic_add_fetch(&g_stamp, 1u, __ATOMIC_RELAXED); while (p.stamp == 0u);  // 0 means "cleared"
+        if (!p.dry) do p.stamp = __atomic_add_fetch(&g_stamp, 1u, __ATOMIC_RELAXED); while (p.stamp == 0u);  // 0 means "cleared"
         return i8 ? launch_gemm_i8(p, cfg, fold, 2, st) : launch_gemm_f8(p, cfg, fold, 2, st);
     }
     if (splits > 1) {
@@ -528,7 +562,7 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
         p.vec_store = d->n % 4 == 0;
         p.vec_store16 = 0;
         const int rc = i8 ? launch_gemm_i8(p, cfg, fold, splits, st) : launch_gemm_f8(p, cfg, fold, splits, st);
-        if (rc != SEGQ_OK) return rc;
+        if (rc != SEGQ_OK || p.dry) return rc;
         const bool vec = d->n % 4 == 0 && d->ldo % 4 == 0 && al(d->out, 16);
         const int64_t items = d->m * (vec ? d->n / 4 : d->n);
         const dim3 grid((unsigned)((items + 255) / 256));
@@ -650,26 +684,43 @@ int segq_init(void) {
 
 int64_t segq_noalloc_scratch_bytes(void) { return SCRATCH_BYTES; }
 
+int segq_device_info(int32_t* compute_units, int32_t* max_engine_clock_khz) {
+    int dev = 0, cus = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, dev) != hipSuccess)
+        return fail(SEGQ_ERR_LAUNCH, "segq_device_info: cannot read the current device's attributes");
+    if (compute_units) *compute_units = cus;
+    if (max_engine_clock_khz) *max_engine_clock_khz = khz;
+    return SEGQ_OK;
+}
+
 int segq_gemm_noalloc(const segq_gemm_desc* d, segq_stream_t stream) {
     GemmPlan plan;
     int rc = gemm_impl(d, nullptr, &plan);
     if (rc != SEGQ_OK) return rc;
-    const int64_t need = plan.bytes;
-    if (need > SCRATCH_BYTES)
-        return fail(SEGQ_ERR_ARG, "segq_gemm_noalloc: this launch would use %lld bytes of workspace, the library's scratch "
-                                  "array holds %lld; use segq_gemm with a workspace of the caller's",
-                    (long long)need, (long long)SCRATCH_BYTES);
+    const int64_t wish = plan.bytes;  // what the launch would use of an unlimited workspace
     segq_gemm_desc c = *d;
     c.workspace = nullptr;
     c.workspace_bytes = 0;
-    if (need > 0) {
+    if (wish > 0) {
         void* ptr = nullptr;
         rc = scratch_address(&ptr);  // resolved once per device (segq_init does it ahead of time)
         if (rc != SEGQ_OK) return rc;
         c.workspace = ptr;
         c.workspace_bytes = SCRATCH_BYTES;
     }
-    return gemm_impl(&c, static_cast<hipStream_t>(stream));
+    // a launch that could use more than the array holds runs with what fits, as segq_gemm does with
+    // a workspace of that size (fewer K shares, a second register set instead of parked sums); it
+    // is refused only where it cannot run with less
+    rc = gemm_impl(&c, static_cast<hipStream_t>(stream));
+    if (rc != SEGQ_OK && wish > SCRATCH_BYTES) {
+        char why[256];
+        snprintf(why, sizeof(why), "%s", g_err);
+        return fail(rc, "segq_gemm_noalloc: this launch needs more workspace than the library's scratch array holds (%lld bytes; "
+                        "it could use %lld): %s; use segq_gemm with a workspace of the caller's",
+                    (long long)SCRATCH_BYTES, (long long)wish, why);
+    }
+    return rc;
 }
 
 int segq_linear(const segq_quant_desc* q, const segq_gemm_desc* g, segq_stream_t stream) {

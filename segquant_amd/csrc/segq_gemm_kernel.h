@@ -51,7 +51,7 @@ struct GemmParams {
     int32_t vec_add;      // its rows allow 4-element vector loads
     int32_t pad2_;
     int32_t splits;       // > 1: grid.y workgroups share the K steps of a tile (gemm_pipe_kernel only)
-    int32_t pad_;
+    int32_t rot;          // several ranges, no K split: XCD x starts its walk at range x mod nr (gemm_pipe_kernel only)
     float* park;          // fp32 workspace, one tile-sized slot per workgroup, for finished ranges (or null)
     float* part;          // splits == 2 finished in the launch: two tile-sized fp32 shares per tile (or null)
     unsigned int* arrived;  // ... and one word per tile: the first of the two workgroups leaves `stamp` there
@@ -63,7 +63,15 @@ struct GemmParams {
     const uint16_t* lr_l2;
     int64_t lr_ldt, lr_ldl;  // their row strides in elements
     int32_t lr_rank;         // multiple of 32; 0: no low-rank branch
+    void* oc;                // codes instead of floats: the (M, N) code tensor, or null
+    void* oc_neg;            // DualScale: the second code tensor (Xn), or null
+    int64_t ldoc;            // their row stride in bytes
+    const float* oc_scale;   // one multiplicative scale (x >= 0, or everything when oc_neg is null)
+    const float* oc_scale_neg;
+    int32_t oc_fmt, oc_pre;  // segq_code (I8 / E4M3), segq_pre_op
+    int32_t oc_vec;          // rows allow 8-byte stores
     int32_t pad3_;
+    int32_t dry;             // host only: walk the dispatch down to the kernel instance, launch nothing (segq_gemm_plan)
     KRange r[SEGQ_MAX_RANGES];
 };
 
@@ -98,6 +106,14 @@ __device__ __forceinline__ void add_addend4(const GemmParams& p, int64_t z, int 
         for (int v = 0; v < 4; ++v) o[v] += (p.out_dtype == SEGQ_BF16) ? bf16_bits_to_f32(h[v]) : f16_bits_to_f32(h[v]);
     }
 }
+// acc / (sx sw) + bias as the epilogues evaluate it: the row factor first, then one fused
+// multiply-add with the column factor and the bias.  One definition, no contraction left to the
+// compiler: the epilogue that stores floats and the one that stores codes must round alike.
+__device__ __forceinline__ float dequant_bias(float acc, float rx, float rw, float bias) {
+#pragma clang fp contract(off)
+    return __builtin_fmaf(acc * rx, rw, bias);
+}
+
 constexpr int BK = 128;  // code bytes of K per step
 
 // Chunk swizzle.  The LDS of gfx950 has 64 banks of 4 bytes (a 256-byte span),
@@ -418,7 +434,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
-                else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
+                else o[v] = dequant_bias((float)acc[a][b][v], rx[b], rw[v], bv[v]);
             }
             add_addend4(p, z, m, n, o);
             const int64_t e = c_off + (int64_t)m * p.ldc + n;
@@ -459,6 +475,7 @@ template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>
 int launch_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_kernel<BM, BN, WGM, WGN, FMT, B4, FOLD>;
     constexpr int lds = 2 * (BM + BN) * BK;
+    if (p.dry) return SEGQ_OK;
     static unsigned long long attr_done = 0;
     if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);

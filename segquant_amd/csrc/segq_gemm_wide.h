@@ -18,6 +18,7 @@
 //    LDS patch every store instruction writes four full 256-byte row pieces.
 #pragma once
 #include "segq_gemm_kernel.h"
+#include "segq_encode.h"
 #include <type_traits>
 
 namespace segq {
@@ -57,6 +58,98 @@ __device__ __forceinline__ void store4(void* C, int64_t e, const float (&o)[4], 
     }
 }
 
+
+// Four codes of fmt from four values (already scaled), low byte first.
+__device__ __forceinline__ uint32_t pack4_codes(int fmt, float a, float b, float c, float d) {
+    return fmt == SEGQ_CODE_I8 ? pack4_i8(a, b, c, d) : pack4_e4m3(a, b, c, d);
+}
+
+// The epilogue that writes CODES: what a quantise launch with a static per-tensor scale (or a
+// DualScale pair, two code tensors) and a fused activation function would have made of this
+// GEMM's 16-bit output, bit for bit: the de-quantised sum plus bias (and addend) is rounded to
+// out_dtype, the activation function applied in fp32 and rounded to out_dtype again, then
+// scaled and encoded.  The float output itself is never written to memory: every wave passes
+// 16 rows at a time through its own LDS patch in out_dtype (which is also the transposition that
+// gives each lane eight consecutive columns of one row), reads them back, and stores eight
+// codes per lane.  epi: the tile's vectors parked in LDS, [1/sx BM | 1/sw BN | bias BN].
+template <int BM, int BN, int WGM, int WGN, int FMT>
+__device__ __forceinline__ void codes_epilogue(const GemmParams& p, typename AccT<FMT>::type (&acc)[BN / WGN / 16][BM / WGM / 16],
+                                               uint8_t* smem, int m0, int n0, int wave, int lane, const float* epi) {
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 16, TN = WN / 16;
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    const int m_base = m0 + wm * WM + lrow;
+    const int n_base = n0 + wn * WN + 4 * lgrp;
+    const bool dual = p.oc_neg != nullptr;
+    const float s_pos = p.oc_scale[0];
+    const float s_neg = dual ? p.oc_scale_neg[0] : s_pos;
+    const bool bf = p.out_dtype == SEGQ_BF16;
+    const int dt = p.out_dtype, fmt = p.oc_fmt, op = p.oc_pre;
+    constexpr int RS = WN * 2 + 16;  // patch row stride in bytes; the 16 spreads the rows over the banks
+    constexpr int CH = WN / 8;       // 8-element pieces per patch row
+    __syncthreads();                 // the operand tiles are dead from here on
+    uint8_t* const patch = smem + wave * 16 * RS;
+    uint8_t* const ocp = static_cast<uint8_t*>(p.oc);
+    uint8_t* const ocn = static_cast<uint8_t*>(p.oc_neg);
+    // the 16 rows in the patch -> codes.  A real loop over b would have to index the accumulators, so
+    // the blocks below are unrolled, each followed by this loop
+    auto encode_rows = [&](int b) __attribute__((always_inline)) {
+        for (int j = 0; j < (16 * CH + 63) / 64; ++j) {
+            const int c = j * 64 + lane;
+            const int row = c / CH, col = c % CH;
+            if ((16 * CH) % 64 != 0 && c >= 16 * CH) continue;
+            const uint4 raw = *reinterpret_cast<const uint4*>(patch + row * RS + col * 16);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+            float cp[8], cn[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t h = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+                float t = bf ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+                if (op != SEGQ_PRE_NONE) t = round_to(dt, act_value(op, t));
+                // x >= 0 takes the positive scale; the branch not taken holds code(0)
+                // (segquant/src/real_quant/quantizer.cuh:193-203).  One tensor: one scale for both signs.
+                cp[i] = dual ? (t >= 0.0f ? t * s_pos : 0.0f) : t * s_pos;
+                cn[i] = (t >= 0.0f) ? 0.0f : t * s_neg;
+            }
+            const int mm = m0 + wm * WM + b * 16 + row;
+            const int n = n0 + wn * WN + col * 8;
+            if (mm >= p.M || n >= p.N) continue;
+            const int64_t e = (int64_t)mm * p.ldoc + n;
+            const uint2 vp = make_uint2(pack4_codes(fmt, cp[0], cp[1], cp[2], cp[3]), pack4_codes(fmt, cp[4], cp[5], cp[6], cp[7]));
+            uint2 vn = make_uint2(0u, 0u);
+            if (dual) vn = make_uint2(pack4_codes(fmt, cn[0], cn[1], cn[2], cn[3]), pack4_codes(fmt, cn[4], cn[5], cn[6], cn[7]));
+            if (p.oc_vec && n + 7 < p.N) {
+                *reinterpret_cast<uint2*>(ocp + e) = vp;
+                if (dual) *reinterpret_cast<uint2*>(ocn + e) = vn;
+            } else {
+                const uint64_t bp = ((uint64_t)vp.y << 32) | vp.x, bn = ((uint64_t)vn.y << 32) | vn.x;
+                for (int i = 0; i < 8 && n + i < p.N; ++i) {
+                    ocp[e + i] = (uint8_t)(bp >> (8 * i));
+                    if (dual) ocn[e + i] = (uint8_t)(bn >> (8 * i));
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const float rx = epi[wm * WM + b * 16 + lrow];
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+            const v4f rw = *reinterpret_cast<const v4f*>(epi + BM + wn * WN + a * 16 + 4 * lgrp);
+            const v4f bias = *reinterpret_cast<const v4f*>(epi + BM + BN + wn * WN + a * 16 + 4 * lgrp);
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = dequant_bias((float)acc[a][b][v], rx, rw[v], bias[v]);
+            if (p.addend) add_addend4(p, 0, min(m_base + b * 16, p.M - 1), n_base + a * 16, o);
+            *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
+                make_uint2(bf ? pack2_bf16(o[0], o[1]) : pack2_f16(o[0], o[1]), bf ? pack2_bf16(o[2], o[3]) : pack2_f16(o[2], o[3]));
+        }
+        __builtin_amdgcn_wave_barrier();
+        encode_rows(b);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
 
 // Scale, add bias, round once, store.  16-bit outputs of full tiles go through a
 // per-wave LDS patch so that every store instruction writes whole row pieces.
@@ -107,7 +200,6 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
             }
         return;
     }
-
     const bool is16 = p.out_dtype != SEGQ_F32;
     const bool via_lds = is16 && p.vec_store16 && (n0 + BN <= p.N);
     float rx[TM];
@@ -156,7 +248,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
                     float o[4];
 #pragma unroll
                     for (int v = 0; v < 4; ++v)
-                        o[v] = (FOLD ? accf[a][b][v] : (float)acc[a][b][v] * rx[b] * rwv[a][v]) + bvv[a][v];
+                        o[v] = FOLD ? accf[a][b][v] + bvv[a][v] : dequant_bias((float)acc[a][b][v], rx[b], rwv[a][v], bvv[a][v]);
                     if constexpr (ADD) add_addend4(p, z, min(m_base + b * 16, p.M - 1), n_base + a * 16, o);
                     const bool bf = p.out_dtype == SEGQ_BF16;
                     *reinterpret_cast<uint2*>(patch + lrow * RS + (a * 16 + 4 * lgrp) * 2) =
@@ -199,7 +291,7 @@ __device__ __forceinline__ void wide_epilogue(const GemmParams& p, typename AccT
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 if constexpr (FOLD) o[v] = accf[a][b][v] + bv[v];
-                else o[v] = (float)acc[a][b][v] * rx[b] * rw[v] + bv[v];
+                else o[v] = dequant_bias((float)acc[a][b][v], rx[b], rw[v], bv[v]);
             }
             add_addend4(p, z, m, n, o);
             const int64_t e = c_off + (int64_t)m * p.ldc + n;
@@ -515,8 +607,10 @@ __device__ __forceinline__ void lowrank_accumulate(const GemmParams& p, v4f (&of
 // s_waitcnt immediate for "vmcnt(n) lgkmcnt(0)" on gfx9-family encodings
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }
 
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false,
+          bool CODES = false>  // CODES: the epilogue writes the next linear's codes instead of floats (one range)
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmParams p) {
+    static_assert(!CODES || (!FOLD && !GRP && !PARK && !FINISH), "codes out: plain operands, one range");
     constexpr int NW = WGM * WGN, NT = NW * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 16, TN = WN / 16;
@@ -595,6 +689,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
     }
     const int tile_id = bid;  // names this tile's room in the workspaces
+    // Several ranges, no K split: the workgroups of XCD x walk the ranges starting from range
+    // x mod nr (and wrap), so that at any K step only part of the chip is at a range boundary, where
+    // int8 tiles store their sums to the workspace.  All workgroups of an XCD keep the same order:
+    // they share operand panels through its L2.  The order of a tile's fp32 additions depends on
+    // its XCD only, so a launch gives the same bits every time.  ph(j): the range walked j-th.
+    const int r_off = (FOLD && p.rot) ? (int)(blockIdx.x & 7) % p.nr : 0;
+    auto ph = [&](int j) { const int t = j + r_off; return t >= p.nr ? t - p.nr : t; };
     int tile_m, tile_n;
     {
         const int gsz = p.group_m * p.tiles_n;
@@ -710,11 +811,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         if constexpr (PARK) {
             if (r < r_last) {
                 const int rl = r_last;
-                const float* sx = p.r[r].sx;
-                const float* sw = p.r[r].sw;
-                const float* sx2 = p.r[rl].sx;
-                const float* sw2 = p.r[rl].sw;
-                const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs, rs2 = p.r[rl].sx_rs, cs2 = p.r[rl].sw_cs;
+                const float* sx = p.r[ph(r)].sx;
+                const float* sw = p.r[ph(r)].sw;
+                const float* sx2 = p.r[ph(rl)].sx;
+                const float* sw2 = p.r[ph(rl)].sw;
+                const int rs = p.r[ph(r)].sx_rs, cs = p.r[ph(r)].sw_cs, rs2 = p.r[ph(rl)].sx_rs, cs2 = p.r[ph(rl)].sw_cs;
                 float fx[TM];
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
@@ -749,11 +850,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         if constexpr (FOLD && (F8 || GRP)) {
             auto& facc = [&]() -> auto& { if constexpr (GRP) return accf; else return acc; }();
             if (r < r_last) {  // rescale to the next range's units
-                const float* sx = p.r[r].sx + z * p.bsSx;
-                const float* sw = p.r[r].sw + z * p.bsSw;
-                const float* sx2 = p.r[r + 1].sx + z * p.bsSx;
-                const float* sw2 = p.r[r + 1].sw + z * p.bsSw;
-                const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs, rs2 = p.r[r + 1].sx_rs, cs2 = p.r[r + 1].sw_cs;
+                const float* sx = p.r[ph(r)].sx + z * p.bsSx;
+                const float* sw = p.r[ph(r)].sw + z * p.bsSw;
+                const float* sx2 = p.r[ph(r + 1)].sx + z * p.bsSx;
+                const float* sw2 = p.r[ph(r + 1)].sw + z * p.bsSw;
+                const int rs = p.r[ph(r)].sx_rs, cs = p.r[ph(r)].sw_cs, rs2 = p.r[ph(r + 1)].sx_rs, cs2 = p.r[ph(r + 1)].sw_cs;
                 float fx[TM];
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
@@ -774,9 +875,9 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             }
         }
         if constexpr (ACCF) {
-            const float* sx = p.r[r].sx + z * p.bsSx;
-            const float* sw = p.r[r].sw + z * p.bsSw;
-            const int rs = p.r[r].sx_rs, cs = p.r[r].sw_cs;
+            const float* sx = p.r[ph(r)].sx + z * p.bsSx;
+            const float* sw = p.r[ph(r)].sw + z * p.bsSw;
+            const int rs = p.r[ph(r)].sx_rs, cs = p.r[ph(r)].sw_cs;
             float rx[TM];
 #pragma unroll
             for (int b = 0; b < TM; ++b) rx[b] = __builtin_amdgcn_rcpf(sx[(int64_t)min(m_base + b * 16, p.M - 1) * rs]);
@@ -805,25 +906,25 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     if (p.splits > 1) {
         skip = (int)((int64_t)steps * zy / p.splits);
         steps = (int)((int64_t)steps * (zy + 1) / p.splits) - skip;
-        while (lr + 1 < p.nr && skip >= (p.r[lr].k1 - p.r[lr].k0) / BK) {
-            skip -= (p.r[lr].k1 - p.r[lr].k0) / BK;
+        while (lr + 1 < p.nr && skip >= (p.r[ph(lr)].k1 - p.r[ph(lr)].k0) / BK) {
+            skip -= (p.r[ph(lr)].k1 - p.r[ph(lr)].k0) / BK;
             ++lr;
         }
         r_last = r_begin = lr;
-        for (int left = skip + steps; r_last + 1 < p.nr && left > (p.r[r_last].k1 - p.r[r_last].k0) / BK; ++r_last)
-            left -= (p.r[r_last].k1 - p.r[r_last].k0) / BK;
+        for (int left = skip + steps; r_last + 1 < p.nr && left > (p.r[ph(r_last)].k1 - p.r[ph(r_last)].k0) / BK; ++r_last)
+            left -= (p.r[ph(r_last)].k1 - p.r[ph(r_last)].k0) / BK;
     }
-    const int r_first = lr, k_first = p.r[lr].k0 + skip * BK;
-    int lk = k_first, lk1 = p.r[lr].k1;
-    const uint8_t* la = (p.r[lr].a_sel == 1) ? A2b : Ab;
+    const int r_first = lr, k_first = p.r[ph(lr)].k0 + skip * BK;
+    int lk = k_first, lk1 = p.r[ph(lr)].k1;
+    const uint8_t* la = (p.r[ph(lr)].a_sel == 1) ? A2b : Ab;
     auto advance_load = [&]() {
         lk += BK;
         if (lk >= lk1) {
             ++lr;
             const int rr = min(lr, p.nr - 1);  // past the last range nothing more is loaded
-            lk = p.r[rr].k0;
-            lk1 = (lr < p.nr) ? p.r[rr].k1 : 0x7fffffff;
-            la = (p.r[rr].a_sel == 1) ? A2b : Ab;
+            lk = p.r[ph(rr)].k0;
+            lk1 = (lr < p.nr) ? p.r[ph(rr)].k1 : 0x7fffffff;
+            la = (p.r[ph(rr)].a_sel == 1) ? A2b : Ab;
         }
     };
 
@@ -848,7 +949,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             lslot = (lslot + 1) & 3;
         }
     };
-    const int r_epi = ACCF ? 0 : r_last;  // the range whose units the accumulators end up in
+    const int r_epi = ACCF ? 0 : ph(r_last);  // the range (as the caller numbers them) whose units the accumulators end up in
     float epi_val[EPI_IT];
     const bool want_epi = p.out_dtype != SEGQ_ACC;  // raw accumulators come with no scales at all (null pointers)
 #pragma unroll
@@ -899,7 +1000,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
     // pipe of the whole SIMD (both its waves are in the same phase).  Issued one
     // at a time they never queue.  DMA_ and MORE_ are compile-time so that the
     // steady-state loop body has no branches.
-    int cr = r_first, ck = k_first, ck1 = p.r[r_first].k1;  // the tile being multiplied
+    int cr = r_first, ck = k_first, ck1 = p.r[ph(r_first)].k1;  // the tile being multiplied
     bool dirty = false;  // int32 sums not yet folded into the fp32 set (a split can end inside a range)
     int buf = 0;                                   // its buffer, s % NS
     constexpr int NMF = TM * TN, NRD = TM + TN, NDM = A_IT + B_IT;
@@ -1048,8 +1149,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             if constexpr (FOLD) fold(cr);
             ++cr;
             const int rr = min(cr, p.nr - 1);
-            ck = p.r[rr].k0;
-            ck1 = p.r[rr].k1;
+            ck = p.r[ph(rr)].k0;
+            ck1 = p.r[ph(rr)].k1;
         }
         buf = nbuf;
     };
@@ -1102,8 +1203,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             dirty = false;
             ++cr;
             const int rr = min(cr, p.nr - 1);
-            ck = p.r[rr].k0;
-            ck1 = p.r[rr].k1;
+            ck = p.r[ph(rr)].k0;
+            ck1 = p.r[ph(rr)].k1;
         }
         buf = nbuf;
     };
@@ -1219,6 +1320,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
         v4f none[1][1];
         wide_epilogue<BM, BN, WGM, WGN, GEMM_F8, false, false>(p, accp, none, smem, z, m0, n0, wave, lane, r_epi, epi);
+    } else if constexpr (CODES) {
+        codes_epilogue<BM, BN, WGM, WGN, FMT>(p, acc, smem, m0, n0, wave, lane, epi);
     } else {
         wide_epilogue<BM, BN, WGM, WGN, FMT, false, ACCF>(p, acc, accf, smem, z, m0, n0, wave, lane, r_epi, epi);
     }
@@ -1228,6 +1331,7 @@ template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD, bool AS
 int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
     auto kern = gemm_wide_kernel<BM, BN, WGM, WGN, FMT, B4, FOLD, ASEL>;
     constexpr int lds = 2 * (BM + BN) * BK;
+    if (p.dry) return SEGQ_OK;
     static unsigned long long attr_done = 0;
     if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
@@ -1236,11 +1340,13 @@ int launch_wide_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
 }
 
 // wide tile ids (after the generic ones): 256x256 | 256x128 | 128x256 | 128x128, eight waves each
-template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false>
+template <int BM, int BN, int WGM, int WGN, int FMT, bool FOLD, int NS, bool GRP = false, bool PARK = false, bool FINISH = false,
+          bool CODES = false>
 int launch_pipe_instance(const GemmParams& p, int64_t batch, hipStream_t st) {
-    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK, FINISH>;
+    auto kern = gemm_pipe_kernel<BM, BN, WGM, WGN, FMT, FOLD, NS, GRP, PARK, FINISH, CODES>;
     // the stages, the epilogue's vectors, and the ring of group factors
     constexpr int lds = NS * (BM + BN) * BK + (BM + 2 * BN) * 4 + (GRP ? 4 * BN * 4 : 0);
+    if (p.dry) return SEGQ_OK;
     static unsigned long long attr_done = 0;
     if (const int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds, &attr_done)) return rc;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
@@ -1275,6 +1381,18 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
 #define SEGQ_PIPE1(BM_, BN_, WGM_, WGN_, FOLD_, PARK_)                                                               \
     if (tail) break;                                                                                                 \
     return launch_pipe_instance<BM_, BN_, WGM_, WGN_, FMT, FOLD_, 2, false, PARK_, false>(p, batch, st)
+    if (p.oc) {  // the epilogue writes codes: instances of their own, so that the others carry no trace of it
+        if constexpr (!B4) {
+            if (!asel && !fold && !tail && !p.park) {
+                switch (wcfg) {
+                    case 0: return launch_pipe_instance<256, 256, 4, 2, FMT, false, 2, false, false, false, true>(p, batch, st);
+                    case 3: return launch_pipe_instance<128, 128, (FMT == GEMM_F8 ? 4 : 2), (FMT == GEMM_F8 ? 2 : 4), FMT, false, 2, false, false, false, true>(p, batch, st);
+                }
+            }
+        }
+        return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: out_codes runs on tiles %d and %d with plain 8-bit codes on both sides and one range",
+                    FIRST_WIDE_CFG + 1, FIRST_WIDE_CFG + 4);
+    }
     if constexpr (!B4) {
         constexpr bool F8W = FMT == GEMM_F8;  // the e4m3 schedule wants three or more column blocks per wave
         if (!asel) {  // plain 8-bit operands, both straight to LDS: the software-pipelined kernel

@@ -200,6 +200,11 @@ class SegmentLinear(nn.Module):
         the output) are the hooks for the reference's SmoothQuant division and SVD low-rank
         branch (segquant/optimum/optimizer.py:467-470, :731-740), fused into the same kernels."""
         opt = self.optimizer
+        if pre_op is not None and getattr(opt, "l1s", None) is not None:
+            # a low-rank branch multiplies the layer's input itself: evaluate the activation first
+            x, pre_op, gate = self._activated(x, pre_op, gate), None, None
+        if col_div is not None and getattr(opt, "s", None) is not None:
+            raise RuntimeError("a smoothed layer divides by its own factors: an external col_div is not combined with them")
         if not chunked and opt.fused_available():
             return opt.forward_fused(x, self.bias_data if self.bias else None, pre_op=pre_op, gate=gate,
                                      col_div=col_div, addend=addend)
@@ -222,6 +227,32 @@ class SegmentLinear(nn.Module):
         return res + self.bias_data if self.bias else res
 
 
+    def forward_into(self, nxt: "SegmentLinear", x, pre_op=None):
+        """``nxt(op(self(x)))`` for two chained linears (an MLP's fc1 -> activation -> fc2) with the
+        activation codes of ``nxt`` written by this layer's GEMM epilogue: the epilogue adds the
+        bias, rounds to the layer dtype, applies ``pre_op`` ("gelu_tanh" | "gelu" | "silu" | None),
+        rounds again, and encodes with the static activation scale(s) of ``nxt`` (two code tensors
+        for DualScale), bit for bit what ``nxt``'s quantise kernel would have made of the stored
+        tensor.  Neither this layer's float output is written nor a quantise launch reads it back.
+        Not in the reference, which runs the activation as a torch operator on the full-size tensor
+        and quantises it in a launch of its own (backend/torch/layers/activations.py:52-57 in front
+        of segquant/src/real_quant/real_gemm.cu:700-705).  Layers the epilogue does not serve
+        (dynamic or per-token scales in ``nxt``, several K ranges, smoothing, int4 weights here,
+        fp32 inputs) take the two ordinary forwards."""
+        opt, nopt = self.optimizer, nxt.optimizer
+        if nxt.in_features != self.out_features:
+            raise RuntimeError(f"forward_into: {self.out_features} outputs feed a layer with {nxt.in_features} inputs")
+        if getattr(opt, "writes_codes", None) and opt.writes_codes(x) and getattr(nopt, "accepts_codes", None) and nopt.accepts_codes():
+            spec = nopt.code_spec(x.device, pre_op)
+            q, g, ws = opt.fused_launches(x, self.bias_data if self.bias else None, out_codes=spec)
+            if ops_mod().recording_launches():
+                ops_mod().quantize_launch(q)
+                codes = ops_mod().gemm_launch(g, ws)
+            else:
+                codes = ops_mod().linear(q, g, ws)
+            return nopt.forward_codes(codes, x.shape[:-1], x.dtype, nxt.bias_data if nxt.bias else None)
+        return nxt(self(x), pre_op=pre_op)
+
     def forward_parts(self, parts, pre_ops=None):
         """Forward of an input-segmented layer from the tensors that would have been concatenated
         into its input (one per segment), each optionally still in front of its producer's
@@ -233,10 +264,16 @@ class SegmentLinear(nn.Module):
         the concatenated, activated input."""
         opt = self.optimizer
         pre_ops = list(pre_ops) if pre_ops is not None else [None] * len(parts)
-        if self.seg_mode == "input" and opt.fused_available() and getattr(opt.weight_calibrators[0], "group_size", None) is None:
+        if (self.seg_mode == "input" and opt.fused_available() and getattr(opt, "supports_parts", True)
+                and getattr(opt.weight_calibrators[0], "group_size", None) is None):
             return opt.forward_parts(parts, self.bias_data if self.bias else None, pre_ops)
         acted = [p if op is None else self._activated(p, op, None) for p, op in zip(parts, pre_ops)]
         return self.forward(torch.cat(acted, dim=-1))
+
+
+def ops_mod():
+    from .. import ops
+    return ops
 
 
 def create_segment_linear(input_dtype: DType, weight_dtype: DType, opt: Optimum, calib: Calibrate, in_features,

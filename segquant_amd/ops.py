@@ -329,9 +329,15 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
          batch_stride_sx: int = 0, batch_stride_sw: int = 0, out: Optional[torch.Tensor] = None,
          tile: int = 0, workspace: Optional[torch.Tensor] = None,
          group_dequant: Optional[torch.Tensor] = None, split_k: int = 0,
-         addend: Optional[torch.Tensor] = None, lowrank=None):
+         addend: Optional[torch.Tensor] = None, lowrank=None, out_codes: Optional[dict] = None):
     """The ``segq_gemm_desc`` of a segmented GEMM with fused de-quantisation and bias, its output
     tensor, the launch's description and the tensors the descriptor points into.
+
+    ``out_codes``: ``dict(fmt=, scale=, scale_neg=None, pre_op=None)``: the launch writes the CODES
+    the next linear's quantise step would make of the output (rounded to ``out_dtype``, ``pre_op``
+    applied, static per-tensor ``scale``; with ``scale_neg`` the two DualScale tensors) instead of
+    the floats; the returned "output" is then the code tensor, or the pair (Xp, Xn).  See
+    ``segq_gemm_desc.out_codes``.
 
     ``lowrank``: a pair ``(T, L2T)`` of 16-bit matrices in the output's dtype, (m, r) and (n, r)
     with r a multiple of 32: ``T @ L2T.T`` is added to the result inside the epilogue (the SVD
@@ -348,7 +354,14 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
         tdt = torch.float32 if a_fmt == FMT_E4M3 else torch.int32
     else:
         tdt = out_dtype
-    if out is None:
+    oc = oc_neg = None
+    if out_codes is not None:
+        if raw or batch != 1 or out is not None:
+            raise RuntimeError("out_codes needs a float out_dtype, one problem and no out tensor")
+        oc = torch.empty((m, n), dtype=code_dtype(out_codes["fmt"]), device=a.device)
+        if out_codes.get("scale_neg") is not None:
+            oc_neg = torch.empty_like(oc)
+    elif out is None:
         out = torch.empty((batch, m, n) if batch > 1 else (m, n), dtype=tdt, device=a.device)
     d = L.GemmDesc()
     d.a_fmt = _CODE[a_fmt]; d.b_fmt = _CODE[b_fmt]
@@ -356,8 +369,23 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
     d.m = m; d.n = n
     d.a = a.data_ptr(); d.a_neg = a_neg.data_ptr() if a_neg is not None else None; d.lda = lda
     d.b = b.data_ptr(); d.ldb = ldb
-    d.out = out.data_ptr(); d.ldo = n
-    if batch == 1 and out.dim() == 2:  # a view of a wider buffer (a column slice, padded rows) is written in place
+    d.ldo = n
+    if oc is not None:
+        sc, scn = out_codes["scale"], out_codes.get("scale_neg")
+        _need_cuda(sc, scn)
+        if sc.dtype != torch.float32 or sc.numel() != 1 or (scn is not None and (scn.dtype != torch.float32 or scn.numel() != 1)):
+            raise RuntimeError("out_codes takes one float32 scale (and one for the negative side)")
+        d.out_codes = oc.data_ptr(); d.ld_out_codes = n
+        d.out_codes_neg = oc_neg.data_ptr() if oc_neg is not None else None
+        d.out_scale = sc.data_ptr(); d.out_scale_neg = scn.data_ptr() if scn is not None else None
+        d.out_code_fmt = _CODE[out_codes["fmt"]]
+        pre = out_codes.get("pre_op")
+        if pre is not None and pre not in PRE_OPS:
+            raise RuntimeError(f"pre_op must be one of {sorted(PRE_OPS)}")
+        d.out_pre_op = PRE_OPS[pre] if pre is not None else 0
+    else:
+        d.out = out.data_ptr()
+    if oc is None and batch == 1 and out.dim() == 2:  # a view of a wider buffer (a column slice, padded rows) is written in place
         if out.shape != (m, n) or out.dtype != tdt or (n > 1 and out.stride(1) != 1) or (m > 1 and out.stride(0) < n):
             raise RuntimeError("out must be an (m, n) tensor of the output dtype with contiguous rows")
         if m > 1:
@@ -405,7 +433,10 @@ def gemm_desc(a: torch.Tensor, b: torch.Tensor, ranges: Sequence[Range], *, m: i
         kr.sw = r.sw.data_ptr() if r.sw is not None else None
     info = dict(m=m, n=n, batch=batch, k_alg=sum(r.k_len for r in ranges if r.a_sel in (0, 2)),
                 k_exec=sum(r.k_len for r in ranges), a_fmt=a_fmt, b_fmt=b_fmt)
-    return d, out, info, (a, b, a_neg, bias, workspace, group_dequant, addend, lowrank, out, list(ranges))
+    if oc is not None:
+        out = (oc, oc_neg) if oc_neg is not None else oc
+        info["codes_out"] = True
+    return d, out, info, (a, b, a_neg, bias, workspace, group_dequant, addend, lowrank, out, out_codes, list(ranges))
 
 
 # ---------------------------------------------------------------------------

@@ -269,7 +269,8 @@ class DefaultOptimizer(BaseOptimizer):
             out = ops.linear(q, g, ws)
         return out.view(*x.shape[:-1], out.shape[-1])
 
-    def fused_launches(self, x: torch.Tensor, bias=None, pre_op=None, gate=None, col_div=None, addend=None, fresh=False):
+    def fused_launches(self, x: torch.Tensor, bias=None, pre_op=None, gate=None, col_div=None, addend=None, fresh=False,
+                       out_codes=None):
         """What the fused route enqueues for ``x``, not yet launched: the quantise launch
         (``ops.quantize_desc``), the GEMM that reads its codes (``ops.gemm_desc``, output
         (M, out) in ``x.dtype``) and the workspace this layer lends it (or None).  Callers that
@@ -298,9 +299,15 @@ class DefaultOptimizer(BaseOptimizer):
         x2 = x.reshape(-1, K)
         if not x2.is_contiguous():
             x2 = x2.contiguous()
+        if col_div is not None and plan.get("col_div") is not None:
+            raise RuntimeError("this layer already divides by its own smoothing factors: an external col_div is not combined with them")
         if col_div is None:
             col_div = plan.get("col_div")  # a smoothed layer's own divisors
-        plain = pre_op is None and gate is None and col_div is None and addend is None and "l2t" not in plan
+        if "l2t" in plan and (pre_op is not None or gate is not None):
+            # the low-rank operand T = x (L1 / s) is built from the tensor handed in here, so that
+            # tensor must be the layer's input itself, not what is in front of its activation function
+            raise RuntimeError("a layer with a low-rank branch takes its activated input: apply pre_op / gate before the call")
+        plain = pre_op is None and gate is None and col_div is None and addend is None and "l2t" not in plan and out_codes is None
         if plain:
             hit = plan.setdefault("launches", {}).get((x2.shape[0], x.dtype, None if bias is None else bias.data_ptr()))
             if hit is not None:
@@ -348,7 +355,7 @@ class DefaultOptimizer(BaseOptimizer):
         gdq = plan.get("group_dequant")
         add2 = None if addend is None else addend.reshape(M, N).contiguous()
         kw = dict(m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=x.dtype, lda=K, ldb=ldb, bias=bias, a_neg=codes_neg,
-                  group_dequant=gdq)
+                  group_dequant=gdq, out_codes=out_codes)
         g = None
         if "l2t" in plan:
             # the SVD optimiser's low-rank branch: inside the GEMM's epilogue where the library has a
@@ -399,6 +406,61 @@ class DefaultOptimizer(BaseOptimizer):
                 q=(q[0], q[2]), g=(g[0], g[2]), need=0 if ws is None else need, dyn=dyn, dual=dual, S=S, M=M, N=N, sx_src=sx_src,
                 code_shape=tuple(codes.shape), code_dtype=codes.dtype, out_dtype=x.dtype, static=(pos, neg, bias))
         return q, g, ws
+
+    # ---- chained linears: this layer's GEMM writes the next layer's codes ----------------------
+    def accepts_codes(self) -> bool:
+        """Whether another layer's GEMM can write this layer's activation codes: static per-tensor
+        activation scales (DualScale or not), one K range, no smoothing division or low-rank branch
+        (both act on the float input)."""
+        if not self.fused_available():
+            return False
+        cal = self.input_calibrators[0]
+        one_range = self.seg_mode != "input" or self.chunks == 1
+        plain = getattr(self, "s", None) is None and getattr(self, "l1s", None) is None
+        fa = _FMT[self.kernel_type.split("A", 1)[1]]
+        return bool(one_range and plain and not cal.dynamic and cal.axis is None and fa in (ops.FMT_INT8, ops.FMT_E4M3))
+
+    def code_spec(self, device, pre_op=None) -> dict:
+        """What a producing GEMM needs to write this layer's codes (``ops.gemm_desc(out_codes=...)``)."""
+        plan = self._plan or self._build_plan(device)
+        pos, neg = self._static_sx(plan, device)
+        return dict(fmt=plan["fa"], scale=pos[0], scale_neg=neg[0] if self.dual_scale else None, pre_op=pre_op)
+
+    def writes_codes(self, x: torch.Tensor) -> bool:
+        """Whether this layer's GEMM has the epilogue that writes codes for ``x``: plain 8-bit codes on
+        both sides, one K range in whole 128-byte steps, a 16-bit input dtype, nothing but the bias
+        joining the result."""
+        if not self.fused_available() or x.dtype not in (torch.bfloat16, torch.float16):
+            return False
+        plan = self._plan or self._build_plan(x.device)
+        one_range = (self.seg_mode != "input" or self.chunks == 1) and not self.dual_scale
+        return bool(one_range and plan["fw"] != ops.FMT_INT4 and plan["fa"] != ops.FMT_INT4 and plan["K"] % 128 == 0 and
+                    plan.get("group_dequant") is None and plan.get("col_div") is None and "l2t" not in plan)
+
+    def forward_codes(self, codes, lead_shape, out_dtype, bias=None) -> torch.Tensor:
+        """This layer's GEMM on activation codes another launch has written (one tensor, or the
+        DualScale pair): the second half of :meth:`forward_fused`."""
+        codes, codes_neg = codes if isinstance(codes, tuple) else (codes, None)
+        plan = self._plan or self._build_plan(codes.device)
+        K, N = plan["K"], plan["N"]
+        M = codes.shape[0]
+        pos, neg = self._static_sx(plan, codes.device)
+        ranges = [ops.Range(0, K, pos[0], plan["sw"], 0, 0, plan["sw_cs"])]
+        if self.dual_scale:
+            ranges.append(ops.Range(0, K, neg[0], plan["sw"], 1, 0, plan["sw_cs"]))
+        g = ops.gemm_desc(codes, plan["w"], ranges, m=M, n=N, a_fmt=plan["fa"], b_fmt=plan["fw"], out_dtype=out_dtype, lda=K,
+                          ldb=K // 2 if plan["fw"] == ops.FMT_INT4 else K, bias=bias, a_neg=codes_neg,
+                          group_dequant=plan.get("group_dequant"))
+        ws = None
+        int4 = plan["fw"] == ops.FMT_INT4
+        if M >= 3072 or not int4 or plan.get("group_dequant") is not None:
+            need = plan.setdefault("ws_need", {}).get(M)
+            if need is None:
+                need = plan["ws_need"][M] = ops.gemm_workspace_bytes(g)
+            if need:
+                ws = ops.int4_workspace(codes.device, need)
+        out = ops.gemm_launch(g, ws)
+        return out.view(*lead_shape, N)
 
     def _static_sx(self, plan, device):
         """Calibrated activation scales stacked over the input segments: (pos, neg) for DualScale

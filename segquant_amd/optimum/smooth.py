@@ -159,6 +159,8 @@ class SmoothOptimizer(DefaultOptimizer):
                           bounds=bounds, N=N, K=K, col_div=torch.cat([s.to(device) for s in self.s]).contiguous())
         return self._plan
 
+    supports_parts = False  # SegmentLinear.forward_parts concatenates and takes forward() instead
+
     def forward_parts(self, parts, bias=None, pre_ops=None):
         raise NotImplementedError("smooth / svd layers take the concatenated input")
 

@@ -137,7 +137,7 @@ def config_linears(config: int, M: Optional[int] = None) -> List[LinearSpec]:
     raise ValueError(f"no configuration {config}")
 
 
-def build_layer(spec: LinearSpec, device="cuda:0", real_quant=True, x: Optional[torch.Tensor] = None):
+def build_layer(spec: LinearSpec, device="cuda:0", real_quant=True, x: Optional[torch.Tensor] = None, opt_kwargs=None):
     """A calibrated ``SegmentLinear`` for ``spec`` plus the activation tensor it
     was calibrated on (fp32, CPU)."""
     from .layers.SegmentLinear import SegmentLinear
@@ -154,7 +154,8 @@ def build_layer(spec: LinearSpec, device="cuda:0", real_quant=True, x: Optional[
         input_quant_args={"real_quant": real_quant, "dual_scale": dual, "axis": spec.act_axis,
                           "dynamic": spec.dynamic},
         weight_quant_args={"real_quant": real_quant, "axis": spec.weight_axis,
-                           **({"group_size": spec.weight_group} if spec.weight_group else {})}, device=device)
+                           **({"group_size": spec.weight_group} if spec.weight_group else {})}, opt_kwargs=opt_kwargs,
+        device=device)
     layer.calibrate(x.to(device))
     layer.finish_calibrate()
     return layer, x

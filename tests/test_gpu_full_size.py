@@ -233,14 +233,18 @@ def test_full_size_config5_three_ranges_against_closed_form(ops, M, fmt, lend):
     check(np.arange(M), np.asarray(cols))
 
 
-LAYER_CASES = [(1, None, torch.float32), (2, None, torch.bfloat16), (5, 9216, torch.bfloat16), (5, 1024, torch.bfloat16)]
+LAYER_CASES = [(1, None, torch.float32), (2, None, torch.bfloat16), (3, None, torch.bfloat16), (4, None, torch.bfloat16),
+               (5, 9216, torch.bfloat16), (5, 1024, torch.bfloat16)]
 
 
 @pytest.mark.parametrize("config,M,dtype", LAYER_CASES)
 def test_full_size_layers_against_the_oracle(config, M, dtype):
     """SegmentLinear at the benchmark's own sizes with the library's own tile choice and the layer's
     own workspace lending: configuration 1 (256 tokens, whole output), configuration 2 (4096 tokens:
-    fc1 on the two-workgroup 128 x 128 kernel, fc2 DualScale in two code tensors) and configuration 5
+    fc1 on the two-workgroup 128 x 128 kernel, fc2 DualScale in two code tensors), configuration 3
+    (4608 tokens, per-token dynamic scales, the three FLUX linears on their own tiles), configuration 4
+    (8192 and 2048 tokens: the row quantiser at K = 1280 / 5120, int4 weights expanded into the lent
+    workspace, one factor per group of 128 input channels) and configuration 5
     at 9216 and 1024 tokens (int8 parked, e4m3 rescaled in place, split K), on row and column bands
     against the closed form built by the oracle from the layer's codes and scales
     (element-wise: one rounding to the output dtype plus the accumulation's own error)."""

@@ -1372,3 +1372,82 @@ def test_gemm_smallest_problems(ops, fa, fb):
                 y = ops.gemm(ad, bd, [ops.Range(0, K, sx.to(DEV), sw.to(DEV), 0, 1, 1)], out_dtype=odt, bias=bias.to(DEV), **kw)
                 slack = FP8_ACC_TOL * mag / (sx.numpy()[:, None] * sw.numpy()[None, :]) if fa == O.FMT_E4M3 else 0.0
                 assert (np.abs(_np(y).astype(np.float64) - want) <= tol * np.abs(want) + slack + 1e-30).all(), (M, N, K, tile, odt)
+
+
+@pytest.mark.parametrize("fmt", [O.FMT_INT8, O.FMT_E4M3])
+@pytest.mark.parametrize("op", [None, "gelu_tanh", "silu"])
+@pytest.mark.parametrize("dual", [False, True])
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+def test_gemm_epilogue_writes_the_next_linears_codes(ops, fmt, op, dual, dt):
+    """segq_gemm with out_codes: the epilogue adds the bias, rounds to the layer dtype, applies the
+    activation function, rounds again and encodes with a static scale (DualScale: two tensors)
+    instead of writing floats.  (a) Bit for bit the codes of the two launches it replaces: the same
+    GEMM writing the 16-bit tensor, then segq_quantize with pre_op on it.  (b) Against the oracle:
+    activation + quantize_act(_dual) on the oracle's own output rounded to the dtype; the device's
+    reciprocals (1 ulp in the de-quantisation) and exp2 move a value across a rounding boundary
+    now and then, so codes may differ by one step on a small share of the elements, never by
+    more.  Shapes: whole tiles of both tiles built with this epilogue (explicit ids and the
+    library's choice), and ragged ones."""
+    tdt = TDT[dt]
+    cases = [(256, 384, 256, 0), (512, 512, 128, 11), (384, 1152, 256, 14), (130, 208, 384, 14), (77, 144, 128, 0)]
+    for M, N, K, tile in cases:
+        g = np.random.default_rng(1000 + M + N)
+        if fmt == O.FMT_INT8:
+            a = g.integers(-127, 128, size=(M, K)).astype(np.int8)
+            b = g.integers(-127, 128, size=(N, K)).astype(np.int8)
+        else:
+            a = O.e4m3_encode(g.standard_normal((M, K)).astype(np.float32) * 40)
+            b = O.e4m3_encode(g.standard_normal((N, K)).astype(np.float32) * 40)
+        sx = (g.random(M).astype(np.float32) + 0.5) * (40.0 if fmt == O.FMT_INT8 else 20.0)
+        sw = (g.random(N).astype(np.float32) + 0.5) * 30.0
+        bias = g.standard_normal(N).astype(np.float32) * 0.5
+        ad, bd = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
+        sxd, swd, biasd = (torch.from_numpy(t).to(DEV) for t in (sx, sw, bias))
+        rg = [ops.Range(0, K, sxd, swd, 0, 1, 1)]
+        kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, out_dtype=tdt, lda=K, ldb=K, bias=biasd)
+        # the tensor the layer would have stored, from the same kernel (e4m3 sums depend, in their last
+        # bits, on the order in which a kernel family feeds K to the matrix cores)
+        y16 = ops.gemm(ad, bd, rg, tile=tile or 14, **kw)
+        act = O.activation(_np(y16), op, dtype=dt) if op else _np(y16)
+        lim = 127.0 if fmt == O.FMT_INT8 else 448.0
+        if dual:
+            pa, na = O.dual_amax(act)
+            ps, ns = np.float32(lim / max(pa, 1e-6)), np.float32((128.0 if fmt == O.FMT_INT8 else 448.0) / max(na, 1e-6))
+            sp, sn = torch.tensor([ps], device=DEV), torch.tensor([ns], device=DEV)
+        else:
+            ps = np.float32(lim / np.abs(act).max())
+            sp, sn = torch.tensor([ps], device=DEV), None
+        spec = dict(fmt=fmt, scale=sp, scale_neg=sn, pre_op=op)
+        got = ops.gemm(ad, bd, rg, tile=tile, out_codes=spec, **kw)
+        # (a) the two launches it replaces
+        two = ops.quantize(y16, fmt, sp, sn, dual=dual, two_tensors=dual, pre_op=op)
+        for gc, tc in zip(got if dual else (got,), two if dual else (two,)):
+            assert gc.shape == (M, N) and torch.equal(gc, tc), (M, N, K, tile)
+        # (b) the oracle: the stored tensor is the oracle's output to one rounding unit of the dtype (the
+        # device multiplies by reciprocals where the oracle divides), and the codes are the oracle's
+        # activation + quantize_act(_dual) of that stored tensor.  (Fed with its own output instead, the
+        # oracle lands two e4m3 codes away now and then: one unit of bf16 at x = -5 moves gelu(x) by 10 %.)
+        acc = O.gemm_acc(a, b, fmt, fmt)
+        y = acc / (sx.astype(np.float64)[:, None] * sw.astype(np.float64)[None, :]) + bias[None, :]
+        ulp = 2.0 ** -8 if dt == "bf16" else 2.0 ** -11
+        assert (np.abs(_np(y16).astype(np.float64) - y) <= ulp * np.abs(y) + (2e-4 if fmt == O.FMT_E4M3 else 2e-6) * np.abs(y).max()).all()
+        act_o = act
+        if dual:
+            wp, wn = O.quantize_act_dual(act_o[None], np.float32([ps]), np.float32([ns]), fmt)
+            pairs = ((got[0], wp[0]), (got[1], wn[0]))
+        else:
+            pairs = ((got, O.quantize_act(act_o[None], np.float32([ps]), fmt)[0]),)
+        for gc, want in pairs:
+            gcn = gc.cpu().numpy()
+            if fmt == O.FMT_INT8:
+                d = np.abs(gcn.astype(np.int32) - want.astype(np.int32))
+                assert d.max() <= 1 and (d != 0).mean() <= 4e-3, (M, N, d.max(), (d != 0).mean())
+            else:
+                # (e4m3 keeps three mantissa bits however small the value: the gelus' negative tail, which is
+                # all the Xn tensor holds, lands on a neighbouring code far more often than integer codes do)
+                assert (gcn == want).mean() >= 1 - (8e-2 if op else 0.0)
+                vg, vw = O.e4m3_decode(gcn), O.e4m3_decode(want)
+                assert (np.abs(vg - vw) <= 0.126 * np.abs(vw) + 2.0 ** -9).all()
+    # what the epilogue does not serve is refused, not mis-computed
+    with pytest.raises(RuntimeError, match="out_codes"):
+        ops.gemm(ad, bd, [ops.Range(0, 64, sxd, swd, 0, 1, 1), ops.Range(64, 64, sxd, swd, 0, 1, 1)], out_codes=spec, **kw)

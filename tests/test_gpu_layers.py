@@ -313,6 +313,13 @@ def test_forward_parts_writes_the_concatenation_as_codes(fmt):
     want = layer(torch.cat([attn, mlp_act], dim=1))
     same = layer.forward_parts([attn, mlp_act])
     assert torch.equal(same, want)
+    # ... and that is the oracle's closed form of the layer on the concatenated input (codes of each
+    # part with its own scales, three ranges, one rounding to bf16), not only the library's own answer
+    from _layer_oracle import oracle_layer_output
+    ref = oracle_layer_output(layer, spec, _np32(torch.cat([attn, mlp_act], dim=1)))
+    got = _np32(same).astype(np.float64)
+    bound = 2.0 ** -8 * np.abs(ref) + (1e-3 if fmt == "fpe4m3" else 2e-6) * np.abs(ref).max()
+    assert (np.abs(got - ref) <= bound).all()
     fused = layer.forward_parts([attn, mlp_pre], pre_ops=[None, "gelu_tanh"])
     assert fused.shape == want.shape and fused.dtype == want.dtype
     w32, f32 = want.float(), fused.float()
@@ -377,6 +384,33 @@ def test_smooth_and_svd_layers_fused_route_against_the_oracle(opt_type, fmt, seg
     # the smoothed, split layer is still the linear it replaces (quantisation error only)
     ref = torch.nn.functional.linear(x.to(DEV), w.to(DEV), b.to(DEV))
     assert ((out.float() - ref).norm() / ref.norm()).item() < 0.05
+
+
+@pytest.mark.parametrize("opt_type", ["smooth", "svd"])
+def test_smooth_and_svd_layers_with_a_fused_activation_function(opt_type):
+    """pre_op on a smoothed layer is evaluated inside the quantise kernel (in front of the division by
+    s); on an svd layer the low-rank branch multiplies the ACTIVATED input, so the layer evaluates
+    the activation first.  Either way the result is the layer's forward on op(x) (svd: bit for bit;
+    smooth: to the rounding of the codes, the kernel's exp2 / reciprocal against torch's tanhf), an
+    external col_div is refused, and forward_parts falls back to the concatenated forward."""
+    M, K, N = 200, 512, 384
+    layer, xd, (w, b, x) = _smooth_layer(opt_type, "int8", "input", 2, M, K, N, torch.bfloat16, True, axis=True)
+    pre = (torch.randn(M, K, generator=torch.Generator().manual_seed(5)) * 2).to(torch.bfloat16).to(DEV)
+    act = torch.nn.functional.gelu(pre, approximate="tanh")
+    want = layer(act)
+    got = layer(pre, pre_op="gelu_tanh")
+    if opt_type == "svd":
+        assert torch.equal(got, want)
+    else:
+        w32, g32 = want.float(), got.float()
+        assert (g32 - w32).abs().max().item() <= 2e-2 * w32.abs().max().item()
+    with pytest.raises(RuntimeError, match="col_div"):
+        layer(act, col_div=torch.ones(K, device=DEV))
+    if opt_type == "svd":
+        with pytest.raises(RuntimeError, match="low-rank"):
+            layer.optimizer.fused_launches(pre, layer.bias_data, pre_op="gelu_tanh")
+    parts = [act[:, :K // 2].contiguous(), act[:, K // 2:].contiguous()]
+    assert torch.equal(layer.forward_parts(parts), want)
 
 
 def test_smooth_layer_with_output_segments_takes_the_reference_route():
@@ -449,3 +483,36 @@ def test_one_layer_serves_every_float_input_dtype(config):
         ref = layer(xin.float())           # the same rounded values, fp32 in and out
         err = (out.float() - ref).abs().max().item() / ref.abs().max().item()
         assert err <= ulp + 1e-6, (spec.name, dt, err)
+
+
+@pytest.mark.parametrize("fmt", ["fpe4m3", "int8"])
+def test_chained_linears_write_the_next_layers_codes(fmt):
+    """Config 2's MLP pair (fc1 -> GELU(tanh) -> fc2 with DualScale) through ``forward_into``: fc1's GEMM
+    epilogue writes fc2's two code tensors.  Bit for bit the result of the three launches it
+    replaces (fc1's GEMM writing bf16, fc2's quantise kernel with the GELU fused, fc2's GEMM), which
+    the other tests pin against the oracle; and pairs the epilogue does not serve (an fp32 input)
+    take the two ordinary forwards."""
+    import dataclasses
+    from segquant_amd import workloads as W
+    s1, s2 = W.config_linears(2, M=384)
+    s1, s2 = dataclasses.replace(s1, act=fmt, weight=fmt), dataclasses.replace(s2, act=fmt, weight=fmt)
+    fc1, x = W.build_layer(s1, device=DEV, real_quant=True)
+    xd = x.to(torch.bfloat16).to(DEV)
+    # calibrate fc2 on what it will see: gelu(fc1(x))
+    h = torch.nn.functional.gelu(fc1(xd), approximate="tanh")
+    fc2, _ = W.build_layer(s2, device=DEV, real_quant=True, x=h.float().cpu())
+    assert fc1.optimizer.writes_codes(xd) and fc2.optimizer.accepts_codes()
+    want = fc2(fc1(xd), pre_op="gelu_tanh")
+    got = fc1.forward_into(fc2, xd, pre_op="gelu_tanh")
+    assert got.shape == want.shape and got.dtype == want.dtype and torch.equal(got, want)
+    ref = torch.nn.functional.linear(h.float(), W.make_weight(s2).to(DEV), W.make_bias(s2).to(DEV))
+    assert ((got.float() - ref).norm() / ref.norm()).item() < (0.08 if fmt == "fpe4m3" else 0.03)
+    # the launches: one quantise and one GEMM for fc1, one GEMM for fc2
+    from segquant_amd import ops
+    with ops.record_launches() as log:
+        fc1.forward_into(fc2, xd, pre_op="gelu_tanh")
+        torch.cuda.synchronize()
+    assert [k for k, *_ in log] == ["quantize", "gemm", "gemm"]
+    x32 = x.to(DEV)
+    assert not fc1.optimizer.writes_codes(x32)
+    assert torch.equal(fc1.forward_into(fc2, x32, pre_op="gelu_tanh"), fc2(fc1(x32), pre_op="gelu_tanh"))

@@ -554,3 +554,44 @@ def test_tile_and_share_choice_for_the_benchmark_shapes():
     assert t == 14 and s in (2, 3)
     # the low-rank branch moves to a tile that is built with it
     assert _plan(lib, 4608, 12288, one(3072), I8, lowrank=32)[:2] == (11, 1)
+
+
+def test_plan_refuses_what_the_launch_would_refuse():
+    """segq_gemm_plan walks the launch's own dispatch down to the kernel instance: a descriptor whose
+    launch has no kernel (an explicit tile that is not built for parked ranges or for the low-rank
+    branch, a retired tile id) is refused by the plan with the same status, so callers that probe
+    with the plan (the SVD optimiser does) never meet the refusal at launch time."""
+    import ctypes as C
+    from segquant_amd import _lib as L
+    lib = L.lib()
+    lib.segq_last_error.restype = C.c_char_p
+    I8, F8 = 0, 1
+    c5 = [(0, 3072, 0), (3072, 12288, 0), (3072, 12288, 1)]
+
+    def status(m, n, ranges, fmt, tile, lowrank=0, lend=True):
+        d = L.GemmDesc()
+        d.a_fmt = d.b_fmt = fmt
+        d.out_dtype = d.bias_dtype = 2
+        k = max(b + l for b, l, _ in ranges)
+        d.m, d.n, d.lda, d.ldb, d.ldo, d.batch = m, n, k, k, n, 1
+        d.a, d.a_neg, d.b, d.out = 0x10000000, 0x20000000, 0x30000000, 0x40000000
+        d.n_ranges, d.tile = len(ranges), tile
+        for i, (b, l, sel) in enumerate(ranges):
+            d.ranges[i].k_begin, d.ranges[i].k_len, d.ranges[i].a_sel = b, l, sel
+            d.ranges[i].sx, d.ranges[i].sw = 0x60000000, 0x70000000
+        if lowrank:
+            d.lowrank_t, d.lowrank_l2t, d.lowrank_rank, d.ld_lowrank_t, d.ld_lowrank_l2t = 0x80000000, 0x90000000, lowrank, lowrank, lowrank
+        if lend:
+            d.workspace, d.workspace_bytes = 0xA0000000, 1 << 34
+        t = C.c_int32(0)
+        return lib.segq_gemm_plan(C.byref(d), C.byref(t), None, None)
+
+    assert status(4608, 3072, c5, I8, 16) == 0                 # 288 x 192 parks
+    assert status(4608, 3072, c5, I8, 20) == 2                 # 384 x 192 is built for one int8 range only
+    assert status(4608, 3072, c5, I8, 19) == 2                 # and so is the four-stage 128 x 128 kernel
+    assert status(4608, 3072, c5, F8, 20) == 0                 # e4m3 rescales in place on every tile
+    assert status(4608, 3072, [(0, 3072, 0)], I8, 9) == 2      # retired ids
+    assert status(4608, 3072, [(0, 3072, 0)], I8, 10) == 2
+    assert status(4608, 9216, [(0, 3072, 0)], I8, 15, lowrank=32) == 2   # 192 x 288 has no low-rank finish
+    assert status(4608, 9216, [(0, 3072, 0)], I8, 11, lowrank=32) == 0
+    assert status(4608, 9216, [(0, 3072, 0)], I8, 0, lowrank=32) == 0    # the library's own choice always has a kernel
