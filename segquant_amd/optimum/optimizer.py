@@ -141,6 +141,9 @@ class OptimizerRegistry:
         return c(**kwargs)
 
 
+_MAX_CACHED_TOKEN_COUNTS = 8  # (token count, dtype, bias) entries a layer keeps launch descriptors and buffers for
+
+
 @OptimizerRegistry.register("default")
 class DefaultOptimizer(BaseOptimizer):
     def __init__(self, seg_mode, chunks, chunksizes, weight_manager, input_calibrators, weight_calibrators,
@@ -402,7 +405,13 @@ class DefaultOptimizer(BaseOptimizer):
                 sx_src.append((0, s_))
                 if dual and self.dual_segments[s_]:
                     sx_src.append((1, s_))
-            plan["launches"][(M, x.dtype, None if bias is None else bias.data_ptr())] = dict(
+            # a bounded cache: layers fed with ever-changing token counts would otherwise keep descriptors,
+            # code and scale buffers of every count they have seen.  The oldest entry goes (its buffers
+            # with it) unless a stream capture is under way, whose graph may hold their addresses
+            cache = plan["launches"]
+            if len(cache) >= _MAX_CACHED_TOKEN_COUNTS and not torch.cuda.is_current_stream_capturing():
+                cache.pop(next(iter(cache)))
+            cache[(M, x.dtype, None if bias is None else bias.data_ptr())] = dict(
                 q=(q[0], q[2]), g=(g[0], g[2]), need=0 if ws is None else need, dyn=dyn, dual=dual, S=S, M=M, N=N, sx_src=sx_src,
                 code_shape=tuple(codes.shape), code_dtype=codes.dtype, out_dtype=x.dtype, static=(pos, neg, bias))
         return q, g, ws
@@ -548,7 +557,10 @@ class DefaultOptimizer(BaseOptimizer):
         stream = None
         if not fresh:
             stream = ops._stream(dev)
-            reuse = hit.setdefault("buffers", {}).get(stream)
+            bufs = hit.setdefault("buffers", {})
+            if stream not in bufs and len(bufs) >= 4 and not torch.cuda.is_current_stream_capturing():
+                bufs.pop(next(iter(bufs)))  # streams come and go: keep the buffers of the last few
+            reuse = bufs.get(stream)
             if reuse is not None:  # descriptors, codes and scales of the previous call on this stream
                 qd, gd, result, held = reuse
                 qd.x = x2.data_ptr()

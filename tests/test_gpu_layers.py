@@ -516,3 +516,18 @@ def test_chained_linears_write_the_next_layers_codes(fmt):
     x32 = x.to(DEV)
     assert not fc1.optimizer.writes_codes(x32)
     assert torch.equal(fc1.forward_into(fc2, x32, pre_op="gelu_tanh"), fc2(fc1(x32), pre_op="gelu_tanh"))
+
+
+def test_launch_cache_is_bounded_over_token_counts():
+    """A layer fed with many different token counts keeps launch descriptors and buffers for the
+    last few only, and still computes every one of them right (bit-equal to a fresh layer's)."""
+    from segquant_amd import workloads as W
+    from segquant_amd.optimum import optimizer as opt_mod
+    spec = W.config_linears(3, M=64)[0]
+    layer, x = W.build_layer(spec, device=DEV, real_quant=True)
+    fresh, _ = W.build_layer(spec, device=DEV, real_quant=True)
+    xs = x.to(spec.x_dtype).to(DEV)
+    for m in list(range(16, 64, 4)) + [16, 20]:
+        got = layer(xs[:m])
+        assert torch.equal(got, fresh.optimizer.forward_fused(xs[:m], fresh.bias_data, addend=None).view_as(got))
+        assert len(layer.optimizer._plan["launches"]) <= opt_mod._MAX_CACHED_TOKEN_COUNTS
