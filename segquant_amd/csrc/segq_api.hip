@@ -379,8 +379,12 @@ static int gemm_impl(const segq_gemm_desc* d, hipStream_t st, GemmPlan* plan = n
     // itself and waits on HBM latency: the int8 kernel with four LDS stages keeps three K steps in
     // flight instead of one (256 x 9216 x 1536: 14.8 -> 12.9 us, 512 x 6144 x 3072: 25.5 -> 20.4 us)
     if (d->tile == 0 && cfg == FIRST_WIDE_CFG + 3 && i8 && plain8 && !fold && !groups && !lowrank && wide_ok &&
-        ((d->m + 127) / 128) * ((d->n + 127) / 128) * d->batch <= device_cus() && ktotal / 128 >= 6)
+        ((d->m + 127) / 128) * ((d->n + 127) / 128) * d->batch <= device_cus() && ktotal / 128 >= 6) {
         cfg = FIRST_WIDE_CFG + 8;
+        // ... and where 128 x 96 tiles still fit the CUs once and tile the columns exactly, a third more
+        // workgroups pull from memory, each with four K steps in flight (five stages)
+        if (d->n % 96 == 0 && ((d->m + 127) / 128) * (d->n / 96) * d->batch <= device_cus()) cfg = FIRST_WIDE_CFG + 10;
+    }
     // the 8-wave tiles that exist with the finish in output units (low-rank branch, two-way K split)
     auto tail_tile = [](int c) {
         const int w = c - FIRST_WIDE_CFG;

@@ -461,14 +461,14 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_kernel(const GemmParams p)
 
 // ---- host-side launch of one (format, tile, fold) instance -------------------
 struct TileCfg { int bm, bn, wgm, wgn; };
-constexpr int NUM_TILE_CFG = 20;
+constexpr int NUM_TILE_CFG = 21;
 constexpr int FIRST_BIG_CFG = 8;    // two retired ids (a 4-wave 256 x 256 kernel that no shape profited from)
-constexpr int FIRST_WIDE_CFG = 10;  // eight ids: the 8-wave kernels (segq_gemm_wide.h)
+constexpr int FIRST_WIDE_CFG = 10;  // the 8-wave kernels from here on (segq_gemm_wide.h)
 constexpr TileCfg TILE_CFGS[NUM_TILE_CFG] = {
     {256, 256, 2, 2}, {256, 128, 2, 2}, {128, 128, 2, 2}, {64, 128, 2, 2}, {128, 256, 2, 2},
     {256, 256, 2, 4}, {256, 256, 4, 2}, {256, 128, 4, 2}, {256, 256, 2, 2}, {256, 256, 2, 2},
     {256, 256, 4, 2}, {256, 128, 4, 2}, {128, 256, 2, 4}, {128, 128, 2, 4}, {192, 288, 4, 2}, {288, 192, 2, 4},
-    {256, 192, 4, 2}, {192, 256, 2, 4}, {128, 128, 2, 4}, {384, 192, 4, 2},
+    {256, 192, 4, 2}, {192, 256, 2, 4}, {128, 128, 2, 4}, {384, 192, 4, 2}, {128, 96, 4, 2},
 };
 
 template <int BM, int BN, int WGM, int WGN, int FMT, bool B4, bool FOLD>

@@ -1415,6 +1415,12 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
                     case 9:  // wave tiles of 96 x 96
                         if (tail) break;
                         return launch_pipe_instance<384, 192, 4, 2, FMT, false, 2, false, false, false>(p, batch, st);
+                    case 10:  // 128 x 96, five LDS stages: few tokens, more workgroups with four K steps in flight each
+                        if constexpr (!F8W) {
+                            if (tail) break;
+                            return launch_pipe_instance<128, 96, 4, 2, FMT, false, 5, false, false, false>(p, batch, st);
+                        }
+                        break;
                 }
             } else if constexpr (F8W) {  // fp32 accumulators are rescaled in place: every tile serves several ranges
                 switch (wcfg) {

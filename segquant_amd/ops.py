@@ -259,7 +259,7 @@ def gemm_workspace_bytes(g) -> int:
 
 # tile ids of the 8-wave kernels (segq_gemm_desc.tile) -> rows x columns of the output tile
 TILE_SHAPES = {1: "256x256", 2: "256x128", 3: "128x128", 4: "64x128", 5: "128x256", 6: "256x256", 7: "256x256", 8: "256x128",
-               11: "256x256", 12: "256x128", 13: "128x256", 14: "128x128", 15: "192x288", 16: "288x192", 17: "256x192", 18: "192x256", 19: "128x128", 20: "384x192"}
+               11: "256x256", 12: "256x128", 13: "128x256", 14: "128x128", 15: "192x288", 16: "288x192", 17: "256x192", 18: "192x256", 19: "128x128", 20: "384x192", 21: "128x96"}
 
 
 def gemm_plan(g, workspace: Optional[torch.Tensor] = None) -> dict:

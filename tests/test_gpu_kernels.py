@@ -307,6 +307,7 @@ def test_gemm_raw_accumulators(ops, tile, fa, fb, M, N, K):
 
 
 WIDE_TILES = [11, 12, 13, 14, 15, 16, 17, 18, 20]   # the 8-wave kernels; 15 to 18 and 20 (192x288, 288x192, 256x192, 192x256, 384x192) serve plain 8-bit codes only
+# (19 and 21, the many-stage kernels for few tokens, int8 only: test_gemm_many_stage_tiles_for_few_tokens)
 
 
 def _bf16_ulp(ref):
@@ -374,16 +375,19 @@ def test_gemm_eight_wave_tiles(ops, tile, fa, fb, M, N, K):
     assert (np.abs(got2 - want2) <= 4e-6 * (np.abs(p0) + np.abs(p1) + np.abs(bias.numpy())[None, :]) + slack2).all()
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 2176, 1536), (200, 330, 128), (77, 130, 256), (130, 260, 384), (64, 1152, 768)])
-def test_gemm_four_stage_kernel_for_few_tokens(ops, M, N, K):
-    """Tile 19: the int8 128 x 128 kernel with four LDS stages (the library's own choice when the
-    tiles do not fill the CUs once).  Contractions shorter than, equal to and longer than the
-    number of stages, ragged M and N: raw accumulators exact, the fused fp32 and bf16 epilogues
-    within their rounding of the closed form; what it does not serve is refused."""
+@pytest.mark.parametrize("tile", [19, 21])
+@pytest.mark.parametrize("M,N,K", [(256, 2176, 1536), (200, 330, 128), (77, 130, 256), (130, 260, 384), (64, 1152, 768), (256, 9216, 1536)])
+def test_gemm_many_stage_tiles_for_few_tokens(ops, tile, M, N, K):
+    """Tiles 19 and 21: the int8 128 x 128 kernel with four LDS stages and the 128 x 96 one with five
+    (the library's own choice when the tiles do not fill the CUs once; 128 x 96 where it tiles the
+    columns exactly and still fits the CUs once, as on the 256 x 1536 -> 9216 adaLN shape).
+    Contractions shorter than, equal to and longer than the number of stages, ragged M and N: raw
+    accumulators exact, the fused fp32 and bf16 epilogues within their rounding of the closed form;
+    what they do not serve is refused."""
     fmt = O.FMT_INT8
     a, b = _rand_codes((M, K), fmt, 81), _rand_codes((N, K), fmt, 82)
     ad, bd = _to_dev_codes(a, fmt), _to_dev_codes(b, fmt)
-    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, tile=19)
+    kw = dict(m=M, n=N, a_fmt=fmt, b_fmt=fmt, lda=K, ldb=K, tile=tile)
     ref = O.gemm_acc(a, b, fmt, fmt)
     out = ops.gemm(ad, bd, [ops.Range(0, K, None, None)], out_dtype="acc", **kw)
     assert np.array_equal(out.cpu().numpy().astype(np.int64), ref.astype(np.int64))
@@ -395,9 +399,10 @@ def test_gemm_four_stage_kernel_for_few_tokens(ops, M, N, K):
     assert np.abs(_np(y32).astype(np.float64) - want).max() <= 2e-6 * np.abs(want).max()
     y16 = ops.gemm(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **kw)
     assert (np.abs(y16.float().cpu().numpy().astype(np.float64) - want) <= _bf16_ulp(want)).all()
-    if -(-M // 128) * -(-N // 128) >= 32:  # the library's own choice for such a shape
+    own = 21 if N % 96 == 0 and -(-M // 128) * (N // 96) <= 256 else 19
+    if -(-M // 128) * -(-N // 128) >= 32 and tile == own:  # the library's own choice for such a shape
         gd = ops.gemm_desc(ad, bd, rg, out_dtype=torch.bfloat16, bias=bias.to(DEV), **{**kw, "tile": 0})
-        assert ops.gemm_plan(gd)["tile"] == 19
+        assert ops.gemm_plan(gd)["tile"] == own
         assert torch.equal(ops.gemm_launch(gd, None), y16)
     two = [ops.Range(0, 128, sx.to(DEV), sw.to(DEV), 0, 1, 1), ops.Range(128, K - 128, sx.to(DEV), sw.to(DEV), 0, 1, 1)]
     if K > 128:

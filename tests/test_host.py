@@ -534,8 +534,9 @@ def test_tile_and_share_choice_for_the_benchmark_shapes():
     assert _plan(lib, 4608, 3072, one(12288), I8)[:3] == (16, 1, 0)
     assert _plan(lib, 8192, 8192, one(8192), I8)[:3] == (11, 1, 0)      # 384 does not divide 8192
     assert _plan(lib, 4608, 12288, [(0, 1536, 0), (1536, 1536, 0)], I8)[0] != 20   # int8 with two ranges: not on 384x192
-    # configuration 1: 144 tiles of 128x128 do not fill the CUs: the four-stage kernel; fp32 output (0)
-    assert _plan(lib, 256, 9216, one(1536), I8, out_dtype=0)[:3] == (19, 1, 0)
+    # configuration 1: 144 tiles of 128x128 do not fill the CUs: 192 tiles of 128x96 with five stages; fp32 output (0)
+    assert _plan(lib, 256, 9216, one(1536), I8, out_dtype=0)[:3] == (21, 1, 0)
+    assert _plan(lib, 256, 9216 + 128, one(1536), I8, out_dtype=0)[:3] == (19, 1, 0)   # 96 does not divide the columns: 128x128, four stages
     # configuration 2: fc1 in two whole rounds of 256x192; fc2 (DualScale: two ranges) as 128 tiles in two K shares
     assert _plan(lib, 4096, 6144, one(1536), F8)[:3] == (17, 1, 0)
     t, s, p, need = _plan(lib, 4096, 1536, fc2, F8)
