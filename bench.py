@@ -108,6 +108,9 @@ def main():
     ap.add_argument("--pair", action="store_true",
                     help="config 2 only: also time fc1 -> GELU(tanh) -> fc2 as chained linears (forward_into: fc1's GEMM epilogue writes "
                          "fc2's DualScale codes; no float tensor and no quantise launch between the two GEMMs)")
+    ap.add_argument("--lib", default=None,
+                    help="load this build of the library instead of segquant_amd/libsegq.so (measurement variants made by "
+                         "`make -C segquant_amd/csrc variant`, whose results may be wrong on purpose: timings only)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB -> 256 MiB elementwise copy, the yardstick for HBM byte counters")
     args = ap.parse_args()
@@ -115,6 +118,9 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
     import torch
+    if args.lib:
+        from segquant_amd import _lib as _L
+        _L.LIB_PATH = os.path.abspath(args.lib)
     from segquant_amd import ops, workloads as W
     from segquant_amd._lib import lib
     lib()  # fail loudly if the HIP library is missing
@@ -385,6 +391,16 @@ def main():
         # host time to enqueue one linear (descriptor fill + one library call), from the timed region
         "host_us_per_linear": round((t_host - t0) / (args.steps * len(layers)) * 1e6, 2),
     }
+    if args.lib:
+        out["library"] = args.lib
+    # every GEMM launch of the instrumented pass by linear (events on the launching stream)
+    per_gemm = {}
+    gi = 0
+    for kind, e0, e1, info in log:
+        if kind == "gemm":
+            per_gemm.setdefault(specs[gi % len(specs)].name, []).append(e0.elapsed_time(e1) * 1e3)
+            gi += 1
+    out["roofline"]["per_linear_us"] = {k: round(sum(v) / len(v), 2) for k, v in per_gemm.items()}
     if args.producers and args.config == 5:
         import torch.nn.functional as Fn
         res = []

@@ -1154,6 +1154,24 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
         }
         buf = nbuf;
     };
+    // Measurement hooks (off in the library that ships: `make variant`, see the Makefile): the int8 K loop
+    // with its MFMAs, its fragment reads or its DMA compiled out, barriers and waits in place.  The
+    // results are wrong; the durations say what each of the three costs alone and in pairs.
+#ifdef SEGQ_ABLATE_MFMA
+    constexpr bool abl_mfma = true;
+#else
+    constexpr bool abl_mfma = false;
+#endif
+#ifdef SEGQ_ABLATE_LDS
+    constexpr bool abl_lds = true;
+#else
+    constexpr bool abl_lds = false;
+#endif
+#ifdef SEGQ_ABLATE_DMA
+    constexpr bool abl_dma = true;
+#else
+    constexpr bool abl_dma = false;
+#endif
     auto step_i8 = [&](auto dma_c, auto more_c) __attribute__((always_inline)) {
         constexpr bool DMA_ = decltype(dma_c)::value;
         constexpr bool MORE_ = decltype(more_c)::value;
@@ -1163,8 +1181,8 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
                 const int i = a * TM + b;
-                if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(buf, 1, i / RD_EVERY);
-                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
+                if (i % RD_EVERY == 0 && i / RD_EVERY < NRD && !abl_lds) frag1(buf, 1, i / RD_EVERY);
+                if constexpr (!abl_mfma) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[0][a], fa[0][b], acc[a][b], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         // Tile s+1 must have landed (the NS-2 tiles issued after it may still be in
@@ -1181,12 +1199,12 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_pipe_kernel(const GemmPara
             for (int b = 0; b < TM; ++b) {
                 const int i = a * TM + b;
                 if constexpr (DMA_) {
-                    if (i % DM_EVERY == DM_EVERY - 1 && i / DM_EVERY < NDM) dma1(ap, bp, buf, i / DM_EVERY);
+                    if (i % DM_EVERY == DM_EVERY - 1 && i / DM_EVERY < NDM && !abl_dma) dma1(ap, bp, buf, i / DM_EVERY);
                 }
                 if constexpr (MORE_) {
-                    if (i % RD_EVERY == 0 && i / RD_EVERY < NRD) frag1(nbuf, 0, i / RD_EVERY);
+                    if (i % RD_EVERY == 0 && i / RD_EVERY < NRD && !abl_lds) frag1(nbuf, 0, i / RD_EVERY);
                 }
-                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[1][a], fa[1][b], acc[a][b], 0, 0, 0);
+                if constexpr (!abl_mfma) acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[1][a], fa[1][b], acc[a][b], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         // The reads of the next tile's first half have had most of an MFMA group to
