@@ -1496,7 +1496,10 @@ int launch_wide(const GemmParams& p, int wcfg, bool fold, bool asel, int64_t bat
         }
     }
 #undef SEGQ_WIDE
-    return fail(SEGQ_ERR_UNSUPPORTED, "segq_gemm: no wide kernel %d", wcfg);
+    return fail(SEGQ_ERR_UNSUPPORTED,
+                "segq_gemm: tile %d is not built for this launch (its code format, several ranges, a sign selection, a low-rank "
+                "branch or a K split); tile 0 lets the library choose",
+                FIRST_WIDE_CFG + wcfg + 1);
 }
 
 }  // namespace segq
