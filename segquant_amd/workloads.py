@@ -97,7 +97,7 @@ def segment_bounds(spec: LinearSpec) -> List[int]:
 
 
 def config_linears(config: int, M: Optional[int] = None) -> List[LinearSpec]:
-    """The linears of benchmark configuration 1..5 (shapes as in BASELINE.json)."""
+    """The linears of benchmark configuration 1..5 (the shapes the headline metric is quoted on and its parity cases)."""
     if config == 1:
         return [LinearSpec("adaLN", 1, M or 256, 1536, 9216, chunksizes=[1536] * 6, x_dtype=torch.float32,
                            outlier="x20")]
